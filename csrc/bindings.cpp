@@ -47,7 +47,24 @@ int dllm_skinny_gemm(const void*, long, const void*, void*, long, int, int, int,
                      hipStream_t);
 int dllm_moe_max_tiles(int, int);
 int dllm_moe_ffn(const void*, long, long, int, const int*, const float*, int, int, const void*, const void*, int, int*,
-                 int*, void*, float*, void*, hipStream_t);
+                 int*, void*, float*, void*, int, hipStream_t);
+int dllm_rms_rows(const void*, long, int, const float*, void*, long, int, int, int, float, hipStream_t);
+int dllm_norm_resadd(const void*, long, int, const float*, float*, void*, int, int, float, hipStream_t);
+int dllm_conv_silu(const void*, long, int, const float*, const float*, const void*, const int*, const int*, const int*,
+                   const int*, void*, int, int, int, int, hipStream_t);
+int dllm_selective_scan(const void*, const void*, int, const float*, const float*, const void*, long, int, const float*,
+                        const void*, long, float*, void*, int, const int*, const int*, const int*, const int*, void*, int,
+                        int, int, hipStream_t);
+long dllm_retention_lds(int, int);
+int dllm_retention(const void*, long, int, int, int, int, const float*, int, int, const float*, float*, float,
+                   const int*, const int*, const int*, const int*, void*, int, hipStream_t);
+int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
+int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
+int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
+                         void*, int, hipStream_t);
+int dllm_latent_attention(const void*, const void*, long, int, int, int, int, int, long, const float*, int, const void*,
+                          const int*, int, const int*, const int*, const int*, const int*, const int*, int, float, void*,
+                          hipStream_t);
 int dllm_car_alloc(long, void**);
 int dllm_car_get_handle(void*, char*);
 int dllm_car_handle_size();
@@ -883,8 +900,9 @@ void moe_ffn_tg(torch::Tensor x, torch::Tensor ids, torch::Tensor wts, torch::Te
      "moe_ffn_tg");
 }
 
+// act_mode 0: SwiGLU experts (w13 [E, 2I, H]); 1: squared-ReLU experts without a gate (w13 [E, I, H])
 void moe_ffn(torch::Tensor x, torch::Tensor ids, torch::Tensor wts, torch::Tensor w13, torch::Tensor w2,
-             torch::Tensor out) {
+             torch::Tensor out, int64_t act_mode) {
   check_bf16(x, "x");
   check_i32(ids, "ids");
   check_f32(wts, "wts");
@@ -893,10 +911,12 @@ void moe_ffn(torch::Tensor x, torch::Tensor ids, torch::Tensor wts, torch::Tenso
   check_bf16(out, "out");
   TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && out.is_contiguous(), "x 2-D row-major, out contiguous");
   TORCH_CHECK(w13.dim() == 3 && w2.dim() == 3 && w13.is_contiguous() && w2.is_contiguous(), "w13/w2 [E, N, K]");
-  const int64_t T = x.size(0), H = x.size(1), E = w13.size(0), I = w13.size(1) / 2;
+  TORCH_CHECK(act_mode == 0 || act_mode == 1, "act_mode 0 or 1");
+  const int64_t T = x.size(0), H = x.size(1), E = w13.size(0), I = w13.size(1) / (act_mode ? 1 : 2);
   TORCH_CHECK(w13.size(2) == H && w2.size(0) == E && w2.size(1) == H && w2.size(2) == I, "expert weight shapes");
   TORCH_CHECK(ids.dim() == 2 && ids.size(0) == T && wts.sizes() == ids.sizes(), "ids/wts [T, k]");
   TORCH_CHECK(out.size(0) == T && out.size(1) == H, "out shape");
+  TORCH_CHECK(E <= 64 && H % 32 == 0 && I % 32 == 0 && x.stride(0) % 8 == 0, "E <= 64, H and I multiples of 32");
   const int k = ids.size(1);
   auto iopt = ids.options();
   const int P = (int)(T * k), mt = dllm_moe_max_tiles(P, (int)E);
@@ -906,7 +926,7 @@ void moe_ffn(torch::Tensor x, torch::Tensor ids, torch::Tensor wts, torch::Tenso
   auto y = torch::empty({std::max(P, 1), H}, wts.options());
   ok(dllm_moe_ffn(x.data_ptr(), x.stride(0), T, (int)H, ids.data_ptr<int>(), wts.data_ptr<float>(), k, (int)E,
                   w13.data_ptr(), w2.data_ptr(), (int)I, perm.data_ptr<int>(), tiles.data_ptr<int>(), act.data_ptr(),
-                  y.data_ptr<float>(), out.data_ptr(), stream()),
+                  y.data_ptr<float>(), out.data_ptr(), (int)act_mode, stream()),
      "moe_ffn");
 }
 
@@ -1264,12 +1284,233 @@ void embed_ln(torch::Tensor ids, torch::Tensor word, torch::Tensor pos, torch::T
                    out.data_ptr(), T, S, H, word.size(0), (float)eps, stream()),
      "embed_ln");
 }
+// ---- sequence mixers and the f32 residual stream (csrc/kernels/seqmix.hip, latent.hip).
+// Activations are bf16 or f32; `act_f32` reports which and checks that a tensor is one of the two.
+bool act_f32(const torch::Tensor& t, const char* name) {
+  check_dev(t, name);
+  TORCH_CHECK(t.scalar_type() == torch::kBFloat16 || t.scalar_type() == torch::kFloat32, name, " must be bf16 or f32");
+  return t.scalar_type() == torch::kFloat32;
+}
+void check_rows2d(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 2 && t.stride(1) == 1, name, " must be 2-D with unit column stride");
+}
+struct SeqMeta { int S; const int *qstart, *qlen, *ctx, *rows; };
+SeqMeta seq_meta(const torch::Tensor& qstart, const torch::Tensor& qlen, const torch::Tensor& ctx,
+                 const torch::Tensor& rows, int64_t slots) {
+  for (auto* t : {&qstart, &qlen, &ctx, &rows}) check_i32(*t, "sequence metadata");
+  const int S = qstart.numel();
+  TORCH_CHECK(qlen.numel() == S && ctx.numel() == S && rows.numel() >= S, "sequence metadata lengths");
+  TORCH_CHECK(slots >= 1, "state slots");
+  return {S, qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(), rows.data_ptr<int>()};
+}
+
+void rms_rows(torch::Tensor x, c10::optional<torch::Tensor> w, torch::Tensor y, double eps) {
+  const bool xf = act_f32(x, "x"), yf = act_f32(y, "y");
+  check_rows2d(x, "x");
+  check_rows2d(y, "y");
+  TORCH_CHECK(x.sizes() == y.sizes(), "x / y shapes");
+  const float* wp = nullptr;
+  if (w) {
+    check_f32(*w, "w");
+    TORCH_CHECK(w->numel() == x.size(1), "w length");
+    wp = w->data_ptr<float>();
+  }
+  ok(dllm_rms_rows(x.data_ptr(), x.stride(0), xf, wp, y.data_ptr(), y.stride(0), yf, (int)x.size(0), (int)x.size(1),
+                   (float)eps, stream()),
+     "rms_rows");
+}
+
+void norm_resadd(torch::Tensor y, torch::Tensor w, double eps, torch::Tensor x, c10::optional<torch::Tensor> xl) {
+  const bool f = act_f32(y, "y");
+  check_rows2d(y, "y");
+  check_f32(w, "w");
+  check_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.sizes() == y.sizes() && w.numel() == x.size(1), "x / y / w shapes");
+  void* lp = nullptr;
+  if (xl) {
+    TORCH_CHECK(xl->is_cuda() && xl->scalar_type() == y.scalar_type() && xl->is_contiguous() && xl->sizes() == x.sizes(),
+                "x_lp: contiguous, the dtype of y, the shape of x");
+    lp = xl->data_ptr();
+  }
+  ok(dllm_norm_resadd(y.data_ptr(), y.stride(0), f, w.data_ptr<float>(), x.data_ptr<float>(), lp, (int)x.size(0),
+                      (int)x.size(1), (float)eps, stream()),
+     "norm_resadd");
+}
+
+void causal_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor b, torch::Tensor state, torch::Tensor qstart,
+                      torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor y) {
+  const bool f = act_f32(x, "x");
+  check_rows2d(x, "x");
+  check_f32(w, "w");
+  check_f32(b, "b");
+  TORCH_CHECK(w.dim() == 2, "w [C, K]");
+  const int C = w.size(0), K = w.size(1), T = x.size(0);
+  TORCH_CHECK(x.size(1) >= C && b.numel() == C, "x / b widths");
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == x.scalar_type() && state.is_contiguous() && state.dim() == 3 &&
+                  state.size(1) == K - 1 && state.size(2) == C,
+              "conv state [slots, K - 1, C] in the dtype of x");
+  TORCH_CHECK(y.is_cuda() && y.scalar_type() == x.scalar_type() && y.is_contiguous() && y.dim() == 2 && y.size(0) == T &&
+                  y.size(1) == C,
+              "y [T, C]");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  ok(dllm_conv_silu(x.data_ptr(), x.stride(0), f, w.data_ptr<float>(), b.data_ptr<float>(), state.data_ptr(), m.qstart,
+                    m.qlen, m.ctx, m.rows, y.data_ptr(), T, m.S, C, K, stream()),
+     "causal_conv_silu");
+}
+
+void selective_scan(torch::Tensor xc, torch::Tensor dt_raw, torch::Tensor dt_bias, torch::Tensor A, torch::Tensor dbc,
+                    int64_t dt_rank, torch::Tensor D, torch::Tensor xz, torch::Tensor ssm, torch::Tensor conv,
+                    torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor out) {
+  const bool f = act_f32(xc, "xc");
+  for (auto* t : {&dt_raw, &dbc, &xz, &out, &conv})
+    TORCH_CHECK(t->is_cuda() && t->scalar_type() == xc.scalar_type(), "activations share one dtype");
+  check_f32(dt_bias, "dt_bias");
+  check_f32(A, "A");
+  check_f32(D, "D");
+  check_f32(ssm, "ssm_state");
+  TORCH_CHECK(A.dim() == 2, "A [C, N]");
+  const int C = A.size(0), N = A.size(1), T = xc.size(0);
+  TORCH_CHECK(xc.dim() == 2 && xc.is_contiguous() && xc.size(1) == C, "xc [T, C]");
+  TORCH_CHECK(dt_raw.dim() == 2 && dt_raw.is_contiguous() && dt_raw.size(0) == T && dt_raw.size(1) == C, "dt_raw [T, C]");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == xc.sizes(), "out [T, C]");
+  check_rows2d(dbc, "dbc");
+  check_rows2d(xz, "xz");
+  TORCH_CHECK(dbc.size(0) == T && dt_rank >= 0 && dbc.size(1) >= dt_rank + 2 * N, "dbc [T, dt_rank + 2N]");
+  TORCH_CHECK(xz.size(0) == T && xz.size(1) >= 2 * C, "xz [T, 2C]");
+  TORCH_CHECK(dt_bias.numel() == C && D.numel() == C, "dt_bias / D length");
+  TORCH_CHECK(ssm.dim() == 3 && ssm.size(1) == C && ssm.size(2) == N, "ssm_state [slots, C, N]");
+  TORCH_CHECK(conv.is_contiguous() && conv.dim() == 3 && conv.size(0) == ssm.size(0) && conv.size(2) == C,
+              "conv_state [slots, K - 1, C]");
+  auto m = seq_meta(qstart, qlen, ctx, rows, ssm.size(0));
+  ok(dllm_selective_scan(xc.data_ptr(), dt_raw.data_ptr(), f, dt_bias.data_ptr<float>(), A.data_ptr<float>(),
+                         dbc.data_ptr(), dbc.stride(0), (int)dt_rank, D.data_ptr<float>(), xz.data_ptr(), xz.stride(0),
+                         ssm.data_ptr<float>(), conv.data_ptr(), (int)conv.size(1), m.qstart, m.qlen, m.ctx, m.rows,
+                         out.data_ptr(), m.S, C, N, stream()),
+     "selective_scan");
+}
+
+void retention(torch::Tensor qkvg, int64_t H, int64_t d, int64_t dv, torch::Tensor cos_sin, int64_t rot,
+               torch::Tensor decay, torch::Tensor state, double eps, torch::Tensor pos, torch::Tensor qstart,
+               torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor out) {
+  const bool f = act_f32(qkvg, "qkvg");
+  check_rows2d(qkvg, "qkvg");
+  check_f32(cos_sin, "cos_sin");
+  check_f32(decay, "decay");
+  check_f32(state, "state");
+  check_i32(pos, "positions");
+  const int T = qkvg.size(0);
+  TORCH_CHECK(H >= 1 && d >= 1 && dv >= 1 && qkvg.size(1) >= 2 * H * d + 2 * H * dv, "qkvg [T, 2 H d + 2 H dv]");
+  TORCH_CHECK(cos_sin.dim() == 2 && rot >= 0 && rot % 2 == 0 && rot <= d && cos_sin.size(1) >= rot, "rotation table");
+  TORCH_CHECK(decay.numel() == H, "decay per head");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == d && state.size(3) == dv,
+              "state [slots, H, d, dv]");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == qkvg.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == H * dv,
+              "out [T, H dv]");
+  TORCH_CHECK(dllm_retention_lds((int)d, (int)dv) <= 150 * 1024, "dim x vdim state does not fit the LDS");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  ok(dllm_retention(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, cos_sin.data_ptr<float>(),
+                    (int)cos_sin.size(1), (int)rot, decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps, m.qstart,
+                    m.qlen, m.ctx, m.rows, out.data_ptr(), m.S, stream()),
+     "retention");
+}
+
+void relu2_scale(torch::Tensor x, c10::optional<torch::Tensor> gate, int64_t ff, torch::Tensor y) {
+  const bool f = act_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && y.is_cuda() && y.scalar_type() == x.scalar_type() && y.is_contiguous() &&
+                  y.sizes() == x.sizes(),
+              "x / y contiguous [T, n]");
+  const float* gp = nullptr;
+  int E = 0;
+  if (gate) {
+    check_f32(*gate, "gate");
+    TORCH_CHECK(gate->dim() == 2 && gate->size(0) == x.size(0) && ff >= 1 && gate->size(1) * ff == x.size(1),
+                "gate [T, n / ff]");
+    gp = gate->data_ptr<float>();
+    E = gate->size(1);
+  }
+  ok(dllm_relu2_scale(x.data_ptr(), f, gp, E, (int)std::max<int64_t>(ff, 1), y.data_ptr(), x.size(0), (int)x.size(1),
+                      stream()),
+     "relu2_scale");
+}
+
+void dense_gate(torch::Tensor ids, torch::Tensor wts, torch::Tensor g) {
+  check_i32(ids, "ids");
+  check_f32(wts, "wts");
+  check_f32(g, "gate");
+  TORCH_CHECK(ids.dim() == 2 && wts.sizes() == ids.sizes() && g.dim() == 2 && g.size(0) == ids.size(0), "ids / wts / gate");
+  ok(dllm_dense_gate(ids.data_ptr<int>(), wts.data_ptr<float>(), g.data_ptr<float>(), ids.size(0), (int)ids.size(1),
+                     (int)g.size(1), stream()),
+     "dense_gate");
+}
+
+void latent_kv_write(torch::Tensor ckv, int64_t rank, torch::Tensor w, double eps, torch::Tensor pos,
+                     torch::Tensor cos_sin, torch::Tensor slots, torch::Tensor cache) {
+  const bool f = act_f32(ckv, "ckv");
+  check_rows2d(ckv, "ckv");
+  check_f32(w, "norm weight");
+  check_f32(cos_sin, "cos_sin");
+  check_i32(pos, "positions");
+  check_i32(slots, "slots");
+  const int T = ckv.size(0);
+  const int64_t rot = ckv.size(1) - rank;
+  TORCH_CHECK(rank >= 1 && rot >= 0 && rot % 2 == 0 && w.numel() == rank, "latent / rotated widths");
+  TORCH_CHECK(cos_sin.dim() == 2 && cos_sin.size(1) >= rot, "rotation table");
+  TORCH_CHECK(pos.numel() == T && slots.numel() == T, "positions / slots length");
+  TORCH_CHECK(cache.is_cuda() && cache.scalar_type() == ckv.scalar_type() && cache.is_contiguous() && cache.dim() == 3 &&
+                  cache.size(1) == 16 && cache.size(2) == rank + rot,
+              "cache [blocks, 16, rank + rot] in the dtype of ckv");
+  ok(dllm_latent_kv_write(ckv.data_ptr(), ckv.stride(0), f, (int)rank, (int)rot, w.data_ptr<float>(), (float)eps,
+                          pos.data_ptr<int>(), cos_sin.data_ptr<float>(), (int)cos_sin.size(1), slots.data_ptr<int>(),
+                          cache.data_ptr(), T, stream()),
+     "latent_kv_write");
+}
+
+void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t rot, torch::Tensor pos, torch::Tensor cos_sin,
+                      torch::Tensor cache, torch::Tensor bt, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
+                      torch::Tensor tile_seq, torch::Tensor tile_tok0, double scale, torch::Tensor out) {
+  const bool f = act_f32(qa, "qa");
+  TORCH_CHECK(qa.dim() == 3 && qa.is_contiguous(), "qa [H, T, rank] contiguous");
+  const int64_t H = qa.size(0), T = qa.size(1), rank = qa.size(2);
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == qa.scalar_type(), "q dtype");
+  check_rows2d(q, "q");
+  TORCH_CHECK(q.size(0) == T && q.size(1) >= H * (dim + rot), "q [T, H (dim + rot)]");
+  check_f32(cos_sin, "cos_sin");
+  check_i32(pos, "positions");
+  for (auto* t : {&bt, &qstart, &qlen, &ctx, &tile_seq, &tile_tok0}) check_i32(*t, "attention metadata");
+  TORCH_CHECK(cos_sin.dim() == 2 && rot >= 0 && rot % 2 == 0 && cos_sin.size(1) >= rot, "rotation table");
+  TORCH_CHECK(cache.is_cuda() && cache.scalar_type() == qa.scalar_type() && cache.is_contiguous() && cache.dim() == 3 &&
+                  cache.size(1) == 16 && cache.size(2) == rank + rot,
+              "cache [blocks, 16, rank + rot]");
+  TORCH_CHECK(bt.dim() == 2 && qstart.numel() == bt.size(0) && qlen.numel() == bt.size(0) && ctx.numel() == bt.size(0),
+              "block tables [S, max_blocks] and per-sequence metadata");
+  TORCH_CHECK(tile_tok0.numel() == tile_seq.numel(), "tile tables");
+  TORCH_CHECK(rank <= 512, "latent rank <= 512");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == qa.scalar_type() && out.is_contiguous() && out.sizes() == qa.sizes(),
+              "out like qa");
+  ok(dllm_latent_attention(qa.data_ptr(), q.data_ptr(), q.stride(0), f, (int)H, (int)dim, (int)rot, (int)rank, T,
+                           cos_sin.data_ptr<float>(), (int)cos_sin.size(1), cache.data_ptr(), bt.data_ptr<int>(),
+                           (int)bt.size(1), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
+                           tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), (float)scale,
+                           out.data_ptr(), stream()),
+     "latent_attention");
+}
 }  // namespace
 
 PYBIND11_MODULE(_hip_kernels, m) {
+  m.def("rms_rows", &rms_rows);
+  m.def("norm_resadd", &norm_resadd);
+  m.def("causal_conv_silu", &causal_conv_silu);
+  m.def("selective_scan", &selective_scan);
+  m.def("retention", &retention);
+  m.def("relu2_scale", &relu2_scale);
+  m.def("dense_gate", &dense_gate);
+  m.def("latent_kv_write", &latent_kv_write);
+  m.def("latent_attention", &latent_attention);
   m.def("encoder_attention", &encoder_attention);
   m.def("embed_ln", &embed_ln);
-  m.def("moe_ffn", &moe_ffn);
+  m.def("moe_ffn", &moe_ffn, py::arg("x"), py::arg("ids"), py::arg("wts"), py::arg("w13"), py::arg("w2"), py::arg("out"),
+        py::arg("act_mode") = 0);
   m.def("moe_ffn_tg", &moe_ffn_tg);
   m.def("tgemm", &tgemm);
   m.def("res_add_ssq", &res_add_ssq);

@@ -1,0 +1,252 @@
+// Latent attention: softmax attention whose keys and values are one shared compressed vector per
+// token (a normed latent of `rank` dims plus a rotated key part of `rot` dims that every head
+// shares).  The per-head key up-projection is absorbed into the query on the host side, so a row
+// (token, head) scores key j as  q_lat . c_j + q_rot . kr_j  and returns  sum_j p_j c_j  (the value
+// up-projection follows as a per-head batched GEMM).  Only [c_j | kr_j] is cached, paged in
+// 16-token blocks.
+//
+//   latent_kv_write   one wave per token: RMS-norm the latent (f32), rotate the shared key part
+//                     (interleaved pairs), write both into the token's cache slot
+//   latent_attention  one workgroup per 16 rows (token-major (token, head) rows of one sequence):
+//                     the rows' queries staged once in LDS as f32 (rotation and the score scale
+//                     applied while staging); keys walk in tiles staged in LDS as f32;
+//                     phase 1: a lane owns a key and sums q . k over the dims (q read as LDS
+//                     broadcasts, k with an odd row stride: no bank conflicts) -> f32 scores, causal
+//                     mask, online softmax per row (wave reductions);
+//                     phase 2: a lane owns latent dims lane, lane + 64, ... and accumulates p . c.
+//                     Each wave owns 4 of the 16 rows through both phases.
+// Activations and the cache are bf16 or f32 (template); scores, softmax and sums are f32.
+#include "common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+template <typename T>
+__global__ void __launch_bounds__(64) latent_kv_write_kernel(const T* __restrict__ ckv, long ld, int rank, int rot,
+                                                             const float* __restrict__ w, float eps,
+                                                             const int* __restrict__ pos,
+                                                             const float* __restrict__ cos_sin, int tab_w,
+                                                             const int* __restrict__ slots, T* __restrict__ cache) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int slot = slots[t];
+  if (slot < 0) return;
+  const T* r = ckv + (long)t * ld;
+  float s = 0.f;
+  for (int i = lane; i < rank; i += 64) { const float v = ldf(r + i); s += v * v; }
+  s = wave_sum(s);
+  const float rs = 1.f / sqrtf(s / (float)rank + eps);
+  T* dst = cache + (long)slot * (rank + rot);
+  for (int i = lane; i < rank; i += 64) stf(dst + i, ldf(r + i) * rs * w[i]);
+  const float* cs = cos_sin + (long)pos[t] * tab_w;
+  const int half = rot >> 1;
+  for (int i = lane; i < half; i += 64) {
+    const float u = ldf(r + rank + 2 * i), v = ldf(r + rank + 2 * i + 1);
+    const float c = cs[i], sn = cs[half + i];
+    stf(dst + rank + 2 * i, u * c - v * sn);
+    stf(dst + rank + 2 * i + 1, v * c + u * sn);
+  }
+}
+
+constexpr int LROWS = 16;
+
+// RI: latent dims per lane in phase 2 (rank <= 64 RI)
+template <typename T, int RI>
+__global__ void __launch_bounds__(256) latent_attention_kernel(
+    const T* __restrict__ qa, const T* __restrict__ q, long ldq, int H, int dim, int rot, int rank, long Ttot,
+    const float* __restrict__ cos_sin, int tab_w, const T* __restrict__ cache, const int* __restrict__ bt, int bt_w,
+    const int* __restrict__ qstart, const int* __restrict__ qlen, const int* __restrict__ ctx,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, T* __restrict__ out, int KT,
+    int tpe) {
+  extern __shared__ float sm[];
+  const int entry = blockIdx.y;
+  const int s = tile_seq[entry];
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int tok0 = tile_tok0[entry];
+  if (tok0 >= n) return;
+  const int ntok = min(tpe, n - tok0);
+  const int nrows = ntok * H;                  // rows of this entry, token-major
+  const int row0 = blockIdx.x * LROWS;
+  if (row0 >= nrows) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  const int Dp = rank + rot, kstride = Dp | 1;
+  float* qsh = sm;                              // [16][Dp]
+  float* ksh = qsh + LROWS * Dp;                // [KT][kstride]
+  float* psh = ksh + KT * kstride;              // [16][64]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = rot >> 1;
+  // stage the rows' queries (f32, scaled): latent part from qa [H, T, rank], rotated part from q
+  for (int e = tid; e < LROWS * Dp; e += 256) {
+    const int rr = e / Dp, c = e % Dp, row = row0 + rr;
+    float v = 0.f;
+    if (row < nrows) {
+      const int tl = tok0 + row / H, h = row % H;
+      const long tok = q0 + tl;
+      if (c < rank) {
+        v = ldf(qa + ((long)h * Ttot + tok) * rank + c);
+      } else {
+        const int i = (c - rank) >> 1;
+        const T* qr = q + tok * ldq + (long)h * (dim + rot) + dim + 2 * i;
+        const float u = ldf(qr), w = ldf(qr + 1);
+        const float* cs = cos_sin + (long)(p0 + tl) * tab_w;
+        v = ((c - rank) & 1) ? w * cs[i] + u * cs[half + i] : u * cs[i] - w * cs[half + i];
+      }
+      v *= scale;
+    }
+    qsh[e] = v;
+  }
+  // causal horizon of the block: the last row's position
+  const int last_row = min(row0 + LROWS, nrows) - 1;
+  const int kmax = p0 + tok0 + last_row / H + 1;
+  int rpos[4];
+  bool rok[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int row = row0 + wave * 4 + a;
+    rok[a] = row < nrows;
+    rpos[a] = p0 + tok0 + (rok[a] ? row / H : 0);
+  }
+  float m[4], l[4], acc[4][RI];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    m[a] = -INFINITY;
+    l[a] = 0.f;
+#pragma unroll
+    for (int i = 0; i < RI; ++i) acc[a][i] = 0.f;
+  }
+  const int* btr = bt + (long)s * bt_w;
+  for (int k0 = 0; k0 < kmax; k0 += KT) {
+    const int nk = min(KT, kmax - k0);
+    __syncthreads();   // the previous tile is consumed (and the queries are staged)
+    for (int e = tid; e < nk * Dp; e += 256) {
+      const int kk = e / Dp, c = e % Dp, kidx = k0 + kk;
+      const long slot = (long)btr[kidx >> 4] * 16 + (kidx & 15);
+      ksh[kk * kstride + c] = ldf(cache + slot * Dp + c);
+    }
+    __syncthreads();
+    // phase 1: lane = key
+    float sc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (lane < nk) {
+      const float* kr = ksh + lane * kstride;
+      const float* qr = qsh + (wave * 4) * Dp;
+      for (int c = 0; c < Dp; ++c) {
+        const float kv = kr[c];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) sc[a] += qr[a * Dp + c] * kv;
+      }
+    }
+    float alpha[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const bool vis = lane < nk && rok[a] && (k0 + lane) <= rpos[a];
+      const float sv = vis ? sc[a] : -INFINITY;
+      const float mn = fmaxf(m[a], wave_max(sv));
+      float p = 0.f;
+      alpha[a] = 1.f;
+      if (mn != -INFINITY) {
+        p = vis ? expf(sv - mn) : 0.f;
+        alpha[a] = expf(m[a] - mn);     // m = -inf -> 0
+        m[a] = mn;
+      }
+      l[a] = l[a] * alpha[a] + wave_sum(p);
+      psh[(wave * 4 + a) * 64 + lane] = p;
+    }
+    __syncthreads();
+    // phase 2: lane = latent dim
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int i = 0; i < RI; ++i) acc[a][i] *= alpha[a];
+    for (int kk = 0; kk < nk; ++kk) {
+      float kv[RI];
+#pragma unroll
+      for (int i = 0; i < RI; ++i) {
+        const int c = lane + 64 * i;
+        kv[i] = c < rank ? ksh[kk * kstride + c] : 0.f;
+      }
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const float p = psh[(wave * 4 + a) * 64 + kk];
+#pragma unroll
+        for (int i = 0; i < RI; ++i) acc[a][i] += p * kv[i];
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int row = row0 + wave * 4 + a;
+    if (row >= nrows) continue;
+    const long tok = q0 + tok0 + row / H;
+    const int h = row % H;
+    const float inv = l[a] > 0.f ? 1.f / l[a] : 0.f;
+#pragma unroll
+    for (int i = 0; i < RI; ++i) {
+      const int c = lane + 64 * i;
+      if (c < rank) stf(out + ((long)h * Ttot + tok) * rank + c, acc[a][i] * inv);
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int dllm_latent_kv_write(const void* ckv, long ld, int f32, int rank, int rot, const float* w, float eps,
+                                    const int* pos, const float* cos_sin, int tab_w, const int* slots, void* cache,
+                                    int T, hipStream_t st) {
+  if (T <= 0) return 0;
+  if (rot < 0 || (rot & 1) || rot > tab_w || rank < 1) return -1;
+  if (f32)
+    hipLaunchKernelGGL(latent_kv_write_kernel<float>, dim3(T), dim3(64), 0, st, (const float*)ckv, ld, rank, rot, w, eps, pos,
+                       cos_sin, tab_w, slots, (float*)cache);
+  else
+    hipLaunchKernelGGL(latent_kv_write_kernel<u16>, dim3(T), dim3(64), 0, st, (const u16*)ckv, ld, rank, rot, w, eps, pos,
+                       cos_sin, tab_w, slots, (u16*)cache);
+  return (int)hipGetLastError();
+}
+
+namespace {
+template <typename T>
+int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T* q, long ldq, int H, int dim, int rot,
+                  int rank, long Ttot, const float* cos_sin, int tab_w, const T* cache, const int* bt, int bt_w,
+                  const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
+                  float scale, T* out, int KT, int tpe) {
+#define LAT(RI)                                                                                                        \
+  do {                                                                                                                 \
+    if (lds > 48 * 1024)                                                                                               \
+      hipFuncSetAttribute((const void*)latent_attention_kernel<T, RI>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
+                          (int)lds);                                                                                   \
+    hipLaunchKernelGGL((latent_attention_kernel<T, RI>), g, dim3(256), lds, st, qa, q, ldq, H, dim, rot, rank, Ttot,   \
+                       cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT, tpe);  \
+  } while (0)
+  if (ri <= 1) LAT(1); else if (ri <= 2) LAT(2); else if (ri <= 4) LAT(4); else LAT(8);
+#undef LAT
+  return (int)hipGetLastError();
+}
+}  // namespace
+
+extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, int f32, int H, int dim, int rot, int rank,
+                                     long Ttot, const float* cos_sin, int tab_w, const void* cache, const int* bt,
+                                     int bt_w, const int* qstart, const int* qlen, const int* ctx, const int* tile_seq,
+                                     const int* tile_tok0, int n_entries, float scale, void* out, hipStream_t st) {
+  if (n_entries <= 0 || Ttot <= 0) return 0;
+  if (rank < 1 || rank > 512 || rot < 0 || (rot & 1) || rot > tab_w || H < 1) return -1;
+  const int Dp = rank + rot, kstride = Dp | 1;
+  int KT = 64;
+  while (KT > 8 && 4L * (LROWS * Dp + (long)KT * kstride + LROWS * 64) > 140 * 1024) KT >>= 1;
+  const long lds = 4L * (LROWS * Dp + (long)KT * kstride + LROWS * 64);
+  if (lds > 150 * 1024) return -2;
+  const int tpe = H >= 16 ? 1 : 16 / H;
+  const dim3 g((tpe * H + LROWS - 1) / LROWS, n_entries);
+  const int ri = (rank + 63) / 64;
+  if (f32)
+    return launch_latent<float>(ri, g, lds, st, (const float*)qa, (const float*)q, ldq, H, dim, rot, rank, Ttot, cos_sin,
+                                tab_w, (const float*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale,
+                                (float*)out, KT, tpe);
+  return launch_latent<u16>(ri, g, lds, st, (const u16*)qa, (const u16*)q, ldq, H, dim, rot, rank, Ttot, cos_sin, tab_w,
+                            (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KT, tpe);
+}

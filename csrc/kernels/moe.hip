@@ -108,6 +108,8 @@ __device__ __forceinline__ bf16x8 ld_or0(const u16* p, bool ok) {
 }
 
 // act[row, c] = silu(x_row . wg_c) * (x_row . wu_c); block = 4 waves x 16 columns, MT rows.
+// ACT 1: experts without a gate projection, act = relu(x_row . w_c)^2 (w13 is then [E, I, H]).
+template <int ACT>
 __global__ void __launch_bounds__(256) moe_gemm13_kernel(const u16* __restrict__ x, long x_stride,
                                                          const int* __restrict__ perm, int k,
                                                          const int* __restrict__ tile_e,
@@ -134,8 +136,8 @@ __global__ void __launch_bounds__(256) moe_gemm13_kernel(const u16* __restrict__
   }
   const int n = col0 + rl;
   const bool nok = n < I;
-  const u16* wg = w13 + ((long)e * 2 * I + (nok ? n : 0)) * H + kq;
-  const u16* wu = wg + (long)I * H;
+  const u16* wg = w13 + ((long)e * (ACT ? 1 : 2) * I + (nok ? n : 0)) * H + kq;
+  const u16* wu = ACT ? wg : wg + (long)I * H;
   f32x4 ag[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   f32x4 au[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
   int kk = 0;
@@ -144,7 +146,7 @@ __global__ void __launch_bounds__(256) moe_gemm13_kernel(const u16* __restrict__
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       bg[s] = ld_or0(wg + kk + 32 * s, nok);
-      bu[s] = ld_or0(wu + kk + 32 * s, nok);
+      if (!ACT) bu[s] = ld_or0(wu + kk + 32 * s, nok);
 #pragma unroll
       for (int g = 0; g < 2; ++g) a[s][g] = ld_or0(arow[g] + kk + 32 * s, aok[g]);
     }
@@ -153,16 +155,16 @@ __global__ void __launch_bounds__(256) moe_gemm13_kernel(const u16* __restrict__
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
         ag[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][g], bg[s], ag[g], 0, 0, 0);
-        au[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][g], bu[s], au[g], 0, 0, 0);
+        if (!ACT) au[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][g], bu[s], au[g], 0, 0, 0);
       }
   }
   for (; kk < H; kk += 32) {
-    const bf16x8 bgs = ld_or0(wg + kk, nok), bus = ld_or0(wu + kk, nok);
+    const bf16x8 bgs = ld_or0(wg + kk, nok), bus = ld_or0(wu + kk, nok && !ACT);
 #pragma unroll
     for (int g = 0; g < 2; ++g) {
       const bf16x8 as = ld_or0(arow[g] + kk, aok[g]);
       ag[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as, bgs, ag[g], 0, 0, 0);
-      au[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as, bus, au[g], 0, 0, 0);
+      if (!ACT) au[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as, bus, au[g], 0, 0, 0);
     }
   }
 #pragma unroll
@@ -172,7 +174,8 @@ __global__ void __launch_bounds__(256) moe_gemm13_kernel(const u16* __restrict__
       const int row = 16 * g + (lane >> 4) * 4 + r;
       if (row < nrows && nok) {
         const float gv = ag[g][r];
-        act[(long)(r0 + row) * I + n] = f2bf(gv / (1.f + __expf(-gv)) * au[g][r]);
+        const float rl = fmaxf(gv, 0.f);
+        act[(long)(r0 + row) * I + n] = f2bf(ACT ? rl * rl : gv / (1.f + __expf(-gv)) * au[g][r]);
       }
     }
 }
@@ -277,15 +280,19 @@ extern "C" int dllm_moe_max_tiles(int P, int E) { return (P + MT - 1) / MT + E; 
 
 extern "C" int dllm_moe_ffn(const void* x, long x_stride, long T, int H, const int* ids, const float* wts, int k,
                             int E, const void* w13, const void* w2, int I, int* perm, int* tiles /*4 x max_tiles*/,
-                            void* act, float* y, void* out, hipStream_t stream) {
+                            void* act, float* y, void* out, int act_mode, hipStream_t stream) {
   if (E < 1 || E > 64 || k < 1 || H % 32 != 0 || I % 32 != 0 || H % 4 != 0) return -1;
   if (T == 0) return 0;
   const int P = (int)(T * k);
   const int max_tiles = (P + MT - 1) / MT + E;
   int *te = tiles, *tr = tiles + max_tiles, *tn = tiles + 2 * max_tiles, *nt = tiles + 3 * max_tiles;
   hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 0, stream, ids, P, E, max_tiles, perm, te, tr, tn, nt);
-  hipLaunchKernelGGL(moe_gemm13_kernel, dim3(max_tiles, (I + 63) / 64), dim3(256), 0, stream, (const u16*)x,
-                     x_stride, perm, k, te, tr, tn, nt, (const u16*)w13, (u16*)act, I, H);
+  if (act_mode)
+    hipLaunchKernelGGL(moe_gemm13_kernel<1>, dim3(max_tiles, (I + 63) / 64), dim3(256), 0, stream, (const u16*)x,
+                       x_stride, perm, k, te, tr, tn, nt, (const u16*)w13, (u16*)act, I, H);
+  else
+    hipLaunchKernelGGL(moe_gemm13_kernel<0>, dim3(max_tiles, (I + 63) / 64), dim3(256), 0, stream, (const u16*)x,
+                       x_stride, perm, k, te, tr, tn, nt, (const u16*)w13, (u16*)act, I, H);
   hipLaunchKernelGGL(moe_gemm2_kernel, dim3(max_tiles, (H + 127) / 128), dim3(256), 0, stream, (const u16*)act, perm,
                      wts, te, tr, tn, nt, (const u16*)w2, y, I, H);
   long n4 = T * (H / 4);

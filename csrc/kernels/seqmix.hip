@@ -1,0 +1,393 @@
+// Sequence mixers beside softmax attention, and the f32 residual stream (gfx950, wave64).
+//
+//   rms_rows         y = x / sqrt(mean(x^2) + eps) (* w): one wave per row, any row length, strided rows
+//   norm_resadd      x (f32) += rmsnorm(y) * w, plus the stream rounded to the model dtype: one
+//                    workgroup per token
+//   conv_silu        short causal convolution per channel + SiLU over a packed batch: token-parallel;
+//                    the inputs before a sequence's first new token come from its state slot
+//   scan             Mamba-1 selective scan: 16 lanes per channel share its states, tokens in order;
+//                    softplus, decay, state and the output gate in f32; refills the convolution state
+//   retention        decayed linear attention: one workgroup per (sequence, head), the [dim x vdim]
+//                    state in LDS, rotate-half positions applied while q / k are staged, unit-RMS
+//                    heads and the SiLU gate in the same launch
+//   relu2_scale      relu(x)^2 (* a per-(token, expert) gate): squared-ReLU experts, dense form
+//   dense_gate       top-k (id, weight) pairs -> [T, E] gate matrix
+//
+// Activations are bf16 or f32 (template T = u16 / float); every sum, state, norm and gate is f32.
+// Sequence metadata: qstart / qlen / ctx / rows per sequence (int32); a sequence with qlen 0 is
+// skipped, one whose first new position (ctx - qlen) is 0 starts from a zero state.
+#include "common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p);
+template <> __device__ __forceinline__ float ldf<u16>(const u16* p) { return bf2f(*p); }
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stf(T* p, float v);
+template <> __device__ __forceinline__ void stf<u16>(u16* p, float v) { *p = f2bf(v); }
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+
+// ---------------------------------------------------------------- rms_rows
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256) rms_rows_kernel(const TI* __restrict__ x, long ldx, const float* __restrict__ w,
+                                                       TO* __restrict__ y, long ldy, int rows, int n, float eps) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const TI* xr = x + (long)row * ldx;
+  float s = 0.f;
+  for (int i = lane; i < n; i += 64) { const float v = ldf(xr + i); s += v * v; }
+  s = wave_sum(s);
+  const float r = 1.f / sqrtf(s / (float)n + eps);
+  TO* yr = y + (long)row * ldy;
+  for (int i = lane; i < n; i += 64) stf(yr + i, ldf(xr + i) * r * (w ? w[i] : 1.f));
+}
+
+// ---------------------------------------------------------------- norm_resadd
+template <typename T>
+__global__ void __launch_bounds__(256) norm_resadd_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ w,
+                                                          float* __restrict__ x, T* __restrict__ xl, int H, float eps) {
+  __shared__ float red[16];
+  const long row = blockIdx.x;
+  const T* yr = y + row * ldy;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) { const float v = ldf(yr + i); s += v * v; }
+  const float r = 1.f / sqrtf(block_sum(s, red) / (float)H + eps);
+  float* xr = x + row * (long)H;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float v = xr[i] + ldf(yr + i) * r * w[i];
+    xr[i] = v;
+    if (xl) stf(xl + row * (long)H + i, v);
+  }
+}
+
+// ---------------------------------------------------------------- causal conv + SiLU
+template <typename T>
+__global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ w,
+                                                        const float* __restrict__ b, const T* __restrict__ state,
+                                                        const int* __restrict__ qstart, const int* __restrict__ qlen,
+                                                        const int* __restrict__ ctx, const int* __restrict__ rows,
+                                                        T* __restrict__ y, int C, int K) {
+  const int s = blockIdx.y;
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+  if (c >= C) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  const T* st = state + (long)rows[s] * (K - 1) * C;
+  const int step = 4 * gridDim.z;
+  const float bias = b[c];
+  for (int j = blockIdx.z * 4 + (threadIdx.x >> 6); j < n; j += step) {
+    float acc = bias;
+    for (int k = 0; k < K; ++k) {
+      const int i = j - (K - 1) + k;
+      float u = 0.f;
+      if (i >= 0) u = ldf(x + (long)(q0 + i) * ldx + c);
+      else if (p0 > 0) u = ldf(st + (long)(K - 1 + i) * C + c);
+      acc += w[c * K + k] * u;
+    }
+    stf(y + (long)(q0 + j) * C + c, silu_f(acc));
+  }
+}
+
+// ---------------------------------------------------------------- selective scan
+// 16 lanes per channel; lane `sub` owns states sub, sub + 16, ... (NS of them).
+template <typename T, int NS>
+__global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, const T* __restrict__ dt_raw,
+                                                   const float* __restrict__ dt_bias, const float* __restrict__ A,
+                                                   const T* __restrict__ dbc, long ldd, int dt_rank,
+                                                   const float* __restrict__ Dv, const T* __restrict__ xz, long ldz,
+                                                   float* __restrict__ ssm, T* __restrict__ conv, int Km1,
+                                                   const int* __restrict__ qstart, const int* __restrict__ qlen,
+                                                   const int* __restrict__ ctx, const int* __restrict__ rows,
+                                                   T* __restrict__ out, int C, int N) {
+  const int s = blockIdx.y;
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int c = blockIdx.x * 16 + (threadIdx.x >> 4), sub = threadIdx.x & 15;
+  if (c >= C) return;   // the 16 lanes of a channel leave together
+  const int q0 = qstart[s], p0 = ctx[s] - n, row = rows[s];
+  float a[NS], S[NS];
+  float* sp = ssm + ((long)row * C + c) * N;
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const int nn = sub + 16 * i;
+    a[i] = nn < N ? A[(long)c * N + nn] : 0.f;
+    S[i] = (nn < N && p0 > 0) ? sp[nn] : 0.f;
+  }
+  const float dtb = dt_bias[c], dd = Dv[c];
+  for (int t = 0; t < n; ++t) {
+    const long tok = q0 + t;
+    const float raw = ldf(dt_raw + tok * C + c) + dtb;
+    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+    const float xv = ldf(xc + tok * C + c);
+    const T* bc = dbc + tok * ldd + dt_rank;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      const int nn = sub + 16 * i;
+      if (nn < N) {
+        S[i] = expf(dt * a[i]) * S[i] + dt * xv * ldf(bc + nn);
+        acc += S[i] * ldf(bc + N + nn);
+      }
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 16);
+    if (sub == 0) {
+      const float z = ldf(xz + tok * ldz + C + c);
+      stf(out + tok * C + c, (acc + dd * xv) * silu_f(z));
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    const int nn = sub + 16 * i;
+    if (nn < N) sp[nn] = S[i];
+  }
+  if (sub == 0 && Km1 > 0) {
+    // the last K-1 inputs of the sequence: new tokens where there are enough, else the slot's older ones
+    T* cs = conv + (long)row * Km1 * C + c;
+    float u[8];
+    for (int k = 0; k < Km1; ++k) {
+      const int i = n - Km1 + k;
+      u[k] = i >= 0 ? ldf(xz + (long)(q0 + i) * ldz + c) : (p0 > 0 ? ldf(cs + (long)(Km1 + i) * C) : 0.f);
+    }
+    for (int k = 0; k < Km1; ++k) stf(cs + (long)k * C, u[k]);
+  }
+}
+
+// ---------------------------------------------------------------- retention
+// One workgroup per (head, sequence).  LDS: state [d][dv], staged q / k (rotated, k scaled) and v of
+// TT tokens, partial sums of the row groups (double-buffered), the TT outputs.
+constexpr int RT_TT = 8;
+
+template <typename T>
+__global__ void __launch_bounds__(256) retention_kernel(const T* __restrict__ qkvg, long ld, int H, int d, int dv,
+                                                        const float* __restrict__ cos_sin, int tab_w, int rot,
+                                                        const float* __restrict__ decay, float* __restrict__ state,
+                                                        float eps, const int* __restrict__ qstart,
+                                                        const int* __restrict__ qlen, const int* __restrict__ ctx,
+                                                        const int* __restrict__ rows, T* __restrict__ out, int LJ) {
+  extern __shared__ float sm[];
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  const int G = 256 / LJ;
+  float* S = sm;                       // [d][dv]
+  float* qs = S + d * dv;              // [TT][d]
+  float* ks = qs + RT_TT * d;          // [TT][d]
+  float* vs = ks + RT_TT * d;          // [TT][dv]
+  float* os = vs + RT_TT * dv;         // [TT][dv]
+  float* part = os + RT_TT * dv;       // [2][G][dv]
+  const int tid = threadIdx.x, j0 = tid % LJ, g = tid / LJ;
+  float* sg = state + ((long)rows[s] * H + h) * d * dv;
+  for (int e = tid; e < d * dv; e += 256) S[e] = p0 > 0 ? sg[e] : 0.f;
+  const float dec = decay[h], kscale = 1.f / sqrtf((float)d);
+  const int half = rot >> 1;
+  const long oq = (long)h * d, ok = (long)H * d + (long)h * d, ov = 2L * H * d + (long)h * dv,
+             og = 2L * H * d + (long)H * dv + (long)h * dv;
+  int buf = 0;
+  for (int t0 = 0; t0 < n; t0 += RT_TT) {
+    const int nt = min(RT_TT, n - t0);
+    __syncthreads();   // the previous tile's outputs are consumed, the state is loaded
+    for (int e = tid; e < nt * d; e += 256) {
+      const int tt = e / d, i = e % d;
+      const T* r = qkvg + (long)(q0 + t0 + tt) * ld;
+      float qv = ldf(r + oq + i), kv = ldf(r + ok + i);
+      if (i < rot) {
+        const int f = i < half ? i : i - half;
+        const float* cs = cos_sin + (long)(p0 + t0 + tt) * tab_w;
+        const float c = cs[f], sn = cs[half + f];
+        const int pi = i < half ? i + half : i - half;
+        const float qp = ldf(r + oq + pi), kp = ldf(r + ok + pi);
+        // pair (u, v) = (x[f], x[f + half]) -> (u c - v s, v c + u s)
+        qv = i < half ? qv * c - qp * sn : qv * c + qp * sn;
+        kv = i < half ? kv * c - kp * sn : kv * c + kp * sn;
+      }
+      qs[e] = qv;
+      ks[e] = kv * kscale;
+    }
+    for (int e = tid; e < nt * dv; e += 256) {
+      const int tt = e / dv, j = e % dv;
+      vs[e] = ldf(qkvg + (long)(q0 + t0 + tt) * ld + ov + j);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float* q = qs + tt * d;
+      const float* k = ks + tt * d;
+      for (int j = j0; j < dv; j += LJ) {
+        const float v = vs[tt * dv + j];
+        float acc = 0.f;
+        for (int i = g; i < d; i += G) {
+          const float sv = dec * S[i * dv + j] + k[i] * v;
+          S[i * dv + j] = sv;
+          acc += sv * q[i];
+        }
+        part[(buf * G + g) * dv + j] = acc;
+      }
+      __syncthreads();
+      for (int j = tid; j < dv; j += 256) {
+        float o = 0.f;
+        for (int gg = 0; gg < G; ++gg) o += part[(buf * G + gg) * dv + j];
+        os[tt * dv + j] = o;
+      }
+      buf ^= 1;
+    }
+    __syncthreads();
+    // unit-RMS head, SiLU gate, store: one wave per token
+    for (int tt = tid >> 6; tt < nt; tt += 4) {
+      const int lane = tid & 63;
+      float ss = 0.f;
+      for (int j = lane; j < dv; j += 64) ss += os[tt * dv + j] * os[tt * dv + j];
+      ss = wave_sum(ss);
+      const float r = 1.f / sqrtf(ss / (float)dv + eps);
+      const long tok = q0 + t0 + tt;
+      for (int j = lane; j < dv; j += 64) {
+        const float gz = ldf(qkvg + tok * ld + og + j);
+        stf(out + tok * ((long)H * dv) + (long)h * dv + j, os[tt * dv + j] * r * silu_f(gz));
+      }
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < d * dv; e += 256) sg[e] = S[e];
+}
+
+// ---------------------------------------------------------------- squared ReLU, dense gate
+template <typename T>
+__global__ void __launch_bounds__(256) relu2_kernel(const T* __restrict__ x, const float* __restrict__ gate, int E,
+                                                    int ff, T* __restrict__ y, long rows, int n) {
+  const long total = rows * (long)n;
+  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < total; e += (long)gridDim.x * 256) {
+    const float v = fmaxf(ldf(x + e), 0.f);
+    float r = v * v;
+    if (gate) r *= gate[(e / n) * E + (int)(e % n) / ff];
+    stf(y + e, r);
+  }
+}
+
+__global__ void __launch_bounds__(256) dense_gate_kernel(const int* __restrict__ ids, const float* __restrict__ wts,
+                                                         float* __restrict__ g, long P, int k, int E) {
+  const long p = (long)blockIdx.x * 256 + threadIdx.x;
+  if (p >= P) return;
+  const int e = ids[p];
+  if (e >= 0 && e < E) g[(p / k) * E + e] = wts[p];   // a token's k experts are distinct
+}
+
+}  // namespace
+
+#define BY_T(f32, call_u16, call_f32) \
+  if (f32) { call_f32; } else { call_u16; }
+
+extern "C" int dllm_rms_rows(const void* x, long ldx, int x_f32, const float* w, void* y, long ldy, int y_f32, int rows,
+                             int n, float eps, hipStream_t st) {
+  if (rows <= 0 || n <= 0) return rows == 0 ? 0 : -1;
+  const dim3 g((rows + 3) / 4), b(256);
+  if (x_f32 && y_f32)
+    hipLaunchKernelGGL((rms_rows_kernel<float, float>), g, b, 0, st, (const float*)x, ldx, w, (float*)y, ldy, rows, n, eps);
+  else if (x_f32)
+    hipLaunchKernelGGL((rms_rows_kernel<float, u16>), g, b, 0, st, (const float*)x, ldx, w, (u16*)y, ldy, rows, n, eps);
+  else if (y_f32)
+    hipLaunchKernelGGL((rms_rows_kernel<u16, float>), g, b, 0, st, (const u16*)x, ldx, w, (float*)y, ldy, rows, n, eps);
+  else
+    hipLaunchKernelGGL((rms_rows_kernel<u16, u16>), g, b, 0, st, (const u16*)x, ldx, w, (u16*)y, ldy, rows, n, eps);
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_norm_resadd(const void* y, long ldy, int f32, const float* w, float* x, void* xl, int rows, int H,
+                                float eps, hipStream_t st) {
+  if (rows <= 0) return rows == 0 ? 0 : -1;
+  BY_T(f32,
+       hipLaunchKernelGGL(norm_resadd_kernel<u16>, dim3(rows), dim3(256), 0, st, (const u16*)y, ldy, w, x, (u16*)xl, H, eps),
+       hipLaunchKernelGGL(norm_resadd_kernel<float>, dim3(rows), dim3(256), 0, st, (const float*)y, ldy, w, x, (float*)xl, H, eps))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_conv_silu(const void* x, long ldx, int f32, const float* w, const float* b, const void* state,
+                              const int* qstart, const int* qlen, const int* ctx, const int* rows, void* y, int T,
+                              int S, int C, int K, hipStream_t st) {
+  if (T <= 0 || S <= 0) return 0;
+  if (K < 1 || K > 9) return -1;
+  int gz = (T + 31) / 32;
+  if (gz > 128) gz = 128;
+  const dim3 g((C + 63) / 64, S, gz), blk(256);
+  BY_T(f32,
+       hipLaunchKernelGGL(conv_silu_kernel<u16>, g, blk, 0, st, (const u16*)x, ldx, w, b, (const u16*)state, qstart, qlen, ctx, rows, (u16*)y, C, K),
+       hipLaunchKernelGGL(conv_silu_kernel<float>, g, blk, 0, st, (const float*)x, ldx, w, b, (const float*)state, qstart, qlen, ctx, rows, (float*)y, C, K))
+  return (int)hipGetLastError();
+}
+
+namespace {
+template <typename T>
+int launch_scan(int ns, dim3 g, hipStream_t st, const T* xc, const T* dt_raw, const float* dt_bias, const float* A,
+                const T* dbc, long ldd, int dt_rank, const float* D, const T* xz, long ldz, float* ssm, T* conv, int Km1,
+                const int* qstart, const int* qlen, const int* ctx, const int* rows, T* out, int C, int N) {
+#define SCAN(NS) hipLaunchKernelGGL((scan_kernel<T, NS>), g, dim3(256), 0, st, xc, dt_raw, dt_bias, A, dbc, ldd, dt_rank, D, xz, ldz, ssm, conv, Km1, qstart, qlen, ctx, rows, out, C, N)
+  if (ns <= 1) SCAN(1); else if (ns <= 2) SCAN(2); else if (ns <= 4) SCAN(4); else SCAN(8);
+#undef SCAN
+  return (int)hipGetLastError();
+}
+}  // namespace
+
+extern "C" int dllm_selective_scan(const void* xc, const void* dt_raw, int f32, const float* dt_bias, const float* A,
+                                   const void* dbc, long ldd, int dt_rank, const float* D, const void* xz, long ldz,
+                                   float* ssm, void* conv, int Km1, const int* qstart, const int* qlen, const int* ctx,
+                                   const int* rows, void* out, int S, int C, int N, hipStream_t st) {
+  if (S <= 0) return 0;
+  if (N < 1 || N > 128 || Km1 < 0 || Km1 > 8) return -1;
+  const int ns = (N + 15) / 16;
+  const dim3 g((C + 15) / 16, S);
+  if (f32)
+    return launch_scan<float>(ns, g, st, (const float*)xc, (const float*)dt_raw, dt_bias, A, (const float*)dbc, ldd, dt_rank,
+                              D, (const float*)xz, ldz, ssm, (float*)conv, Km1, qstart, qlen, ctx, rows, (float*)out, C, N);
+  return launch_scan<u16>(ns, g, st, (const u16*)xc, (const u16*)dt_raw, dt_bias, A, (const u16*)dbc, ldd, dt_rank, D,
+                          (const u16*)xz, ldz, ssm, (u16*)conv, Km1, qstart, qlen, ctx, rows, (u16*)out, C, N);
+}
+
+extern "C" long dllm_retention_lds(int d, int dv) {
+  int lj = 1;
+  while (lj < dv && lj < 64) lj <<= 1;
+  const int G = 256 / lj;
+  return 4L * ((long)d * dv + RT_TT * (2L * d + 2L * dv) + 2L * G * dv);
+}
+
+extern "C" int dllm_retention(const void* qkvg, long ld, int f32, int H, int d, int dv, const float* cos_sin, int tab_w,
+                              int rot, const float* decay, float* state, float eps, const int* qstart, const int* qlen,
+                              const int* ctx, const int* rows, void* out, int S, hipStream_t st) {
+  if (S <= 0) return 0;
+  if (rot < 0 || rot > d || (rot & 1) || rot > tab_w) return -1;
+  const long lds = dllm_retention_lds(d, dv);
+  if (lds > 150 * 1024) return -2;
+  int lj = 1;
+  while (lj < dv && lj < 64) lj <<= 1;
+  const dim3 g(H, S);
+  if (f32) {
+    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(retention_kernel<float>, g, dim3(256), lds, st, (const float*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
+                       decay, state, eps, qstart, qlen, ctx, rows, (float*)out, lj);
+  } else {
+    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(retention_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
+                       decay, state, eps, qstart, qlen, ctx, rows, (u16*)out, lj);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_relu2_scale(const void* x, int f32, const float* gate, int E, int ff, void* y, long rows, int n,
+                                hipStream_t st) {
+  const long total = rows * (long)n;
+  if (total <= 0) return 0;
+  long gr = (total + 255) / 256;
+  if (gr > 8192) gr = 8192;
+  BY_T(f32,
+       hipLaunchKernelGGL(relu2_kernel<u16>, dim3((int)gr), dim3(256), 0, st, (const u16*)x, gate, E, ff, (u16*)y, rows, n),
+       hipLaunchKernelGGL(relu2_kernel<float>, dim3((int)gr), dim3(256), 0, st, (const float*)x, gate, E, ff, (float*)y, rows, n))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_dense_gate(const int* ids, const float* wts, float* g, long T, int k, int E, hipStream_t st) {
+  const long P = T * k;
+  if (P <= 0) return 0;
+  hipLaunchKernelGGL(dense_gate_kernel, dim3((int)((P + 255) / 256)), dim3(256), 0, st, ids, wts, g, P, k, E);
+  return (int)hipGetLastError();
+}

@@ -62,7 +62,9 @@ def build_hip(force: bool = False, jobs: int = 8) -> str:
     os.makedirs(BUILD, exist_ok=True)
     hipcc = _hipcc()
     common = ["-fPIC", "-O3", "-std=c++17", f"--offload-arch={ARCH}", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
-              "-Wno-unused-result", "-Wno-deprecated-declarations"]
+              "-Wno-unused-result", "-Wno-deprecated-declarations",
+              # no packed-f32 VALU forms (device pass only; the host pass warns that it ignores it)
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
     torch_inc = []
     for p in ce.include_paths(device_type="cuda"):

@@ -30,8 +30,9 @@ import numpy as np
 import torch
 
 from .. import ops
-from ..models.configs import ModelConfig, get_model_config
-from ..models.llama import AttnMeta, LlamaModel
+from ..models.configs import HybridConfig, ModelConfig, resolve_config
+from ..models.llama import AttnMeta
+from ..models.registry import build_model
 from ..utils.faults import diag, fault
 from ..parallel.comm import SINGLE, ParallelContext
 from ..utils.tracing import tracer
@@ -132,21 +133,40 @@ class LLMEngine:
     def __init__(self, model: Union[str, ModelConfig], device: str = "cuda", par: ParallelContext = SINGLE,
                  kv_cache_gb: Optional[float] = None, max_num_seqs: int = 256, max_model_len: Optional[int] = None,
                  max_prefill_tokens: int = 16384, prefix_cache: bool = True, use_graphs: bool = True,
-                 seed: int = 0, weights: Optional[str] = None, tokenizer: Optional[str] = None):
-        self.cfg = get_model_config(model) if isinstance(model, str) else model
+                 seed: int = 0, weights: Optional[str] = None, tokenizer: Optional[str] = None,
+                 dtype: torch.dtype = torch.bfloat16, num_kv_blocks: Optional[int] = None):
+        """``model``: a registry name, a model folder (config.json + model.safetensors: its
+        architecture picks the class and the folder is the default ``weights``) or a config.
+        ``dtype``: bfloat16, or float32 for the model classes that run in true 32-bit.
+        ``num_kv_blocks``: an exact paged pool (16-token blocks) instead of ``kv_cache_gb``."""
+        if isinstance(model, str) and os.path.isdir(model) and weights is None:
+            weights = model
+        self.cfg = resolve_config(model)
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None and torch.cuda.is_available():
             # an explicit index: worker threads call torch.cuda.set_device(self.device), which
             # rejects a bare "cuda" (the background loop died on it before serving anything)
             self.device = torch.device("cuda", torch.cuda.current_device())
         self.par = par
-        self.model = LlamaModel(self.cfg, device=self.device, par=par, seed=seed, weights=weights)
+        if dtype != torch.bfloat16 and not isinstance(self.cfg, HybridConfig):
+            raise ValueError(f"{self.cfg.name}: this model class serves bfloat16 only")
+        self.model = build_model(self.cfg, device=self.device, dtype=dtype, par=par, seed=seed, weights=weights)
         self.tok = get_tokenizer(self.cfg.vocab, self.cfg.bos_id, self.cfg.eos_id, tokenizer)
+        if max_model_len is None and isinstance(self.cfg, HybridConfig):
+            max_model_len = 8192           # the design itself has no position limit
         self.max_model_len = min(max_model_len or self.cfg.max_position, self.cfg.max_position)
+        # sequences with recurrent state cannot resume from another request's cached prefix blocks
+        self.recurrent = bool(getattr(self.model, "has_recurrent_state", False))
+        prefix_cache = prefix_cache and not self.recurrent
+        geo = getattr(self.model, "attn_geometry", "llama")
+        self._paged_attn = geo is not None       # softmax attention over paged K/V (split-K work lists)
+        self._nkv = self.model.nkv if self._paged_attn else 1
+        if hasattr(self.model, "ensure_positions"):
+            self.model.ensure_positions(self.max_model_len)
         self.max_num_seqs = max_num_seqs
         self.max_prefill_tokens = max_prefill_tokens
         self.max_blocks = (self.max_model_len + BS - 1) // BS
-        self._alloc_kv(kv_cache_gb)
+        self._alloc_kv(kv_cache_gb, num_kv_blocks)
         self.bm = _need_runtime().BlockManager(self.num_blocks, BS, prefix_cache, int(self.KV_PLACEMENT))
         self._ids = itertools.count()
         self._lock = threading.Lock()          # held by the thread currently driving the step loop
@@ -181,6 +201,8 @@ class LLMEngine:
             self._autotune()      # DLLM_AUTOTUNE=0: heuristic GEMM plans (multi-process tests on one GPU)
         self._graphs: Dict[int, torch.cuda.CUDAGraph] = {}
         self._graph_pool = None
+        self.d_logits: Optional[torch.Tensor] = None    # [max bucket, vocab] f32, kept by feed()
+        self._streams: Dict[object, _Seq] = {}           # forced-token requests by caller key (feed)
         self.collective_trips = 0
         self.trip_steps: List[int] = []   # decode-step counter at each collective trip
         self._check_graph_collectives()
@@ -191,9 +213,10 @@ class LLMEngine:
         # (answers detokenised under the next step); caller-side: encode (submit), output (results)
 
     # ------------------------------------------------------------------ setup
-    def _alloc_kv(self, kv_cache_gb: Optional[float]) -> None:
+    def _alloc_kv(self, kv_cache_gb: Optional[float], num_kv_blocks: Optional[int] = None) -> None:
         m, L = self.model, self.cfg.n_layers
-        per_block = L * 2 * m.nkv * BS * m.d * 2
+        own = hasattr(m, "alloc_caches")     # the model lays out its own paged tensors and state slots
+        per_block = max(1, m.block_bytes(BS)) if own else L * 2 * m.nkv * BS * m.d * 2
         if kv_cache_gb is None:
             if self.device.type == "cuda":
                 free, _ = torch.cuda.mem_get_info(self.device)
@@ -209,6 +232,12 @@ class LLMEngine:
             kv_cache_gb = min(float(kv_cache_gb), max(0.5, free / 2**30 - KV_RESERVE_GB))
         self.kv_cache_gb = float(kv_cache_gb)
         self.num_blocks = max(int(kv_cache_gb * 2**30) // per_block, self.max_blocks + 8)
+        if num_kv_blocks is not None:
+            self.num_blocks = int(num_kv_blocks)
+        if own:
+            # one state slot per batch row (+ the dummy row of padding tiles)
+            self.kv_caches = m.alloc_caches(self.num_blocks, BS, self.max_num_seqs + 1)
+            return
         self.k_cache = torch.empty((L, self.num_blocks, m.nkv, BS, m.d), dtype=m.dtype, device=self.device)
         self.v_cache = torch.empty((L, self.num_blocks, m.nkv, m.d, BS), dtype=m.dtype, device=self.device)
         self.kv_caches = [(self.k_cache[i], self.v_cache[i]) for i in range(L)]
@@ -287,14 +316,15 @@ class LLMEngine:
         self._src_bufs = [torch.zeros(mb, dtype=torch.int64, pin_memory=pin) for _ in range(2)]
         self._out_evts = [torch.cuda.Event() for _ in range(2)] if self.on_gpu else None
         self.d_hidden = torch.zeros((mb, self.cfg.hidden), dtype=self.model.dtype, device=self.device)
-        nkv, dh = self.model.nkv, self.model.d
+        nkv, dh = (self.model.nkv, self.model.d) if self._paged_attn else (1, 1)
+        self.d_rows = torch.arange(R + 1, dtype=torch.int32, device=self.device)   # decode: state slot = row
         self.max_splits = 16
         ws = mb * nkv * self.max_splits * 16
         self.dec_ws = (torch.empty(ws * dh, dtype=torch.float32, device=self.device),
                        torch.empty(ws * 2, dtype=torch.float32, device=self.device),
                        torch.zeros(mb * nkv + 2, dtype=torch.int32, device=self.device))
         # persistent decode attention: host-built work list, copied with the step's metadata
-        self.attn_worklist = self.ATTN_WORKLIST and not self.ATTN_DYNAMIC
+        self.attn_worklist = self.ATTN_WORKLIST and not self.ATTN_DYNAMIC and self._paged_attn
         if self.attn_worklist:
             cap = 4 + 4 * mb * nkv * self.max_splits   # extended list (ops.decode_work_items)
             self._items_bufs = []
@@ -307,6 +337,8 @@ class LLMEngine:
     def _autotune(self) -> None:
         """Pick the fastest GEMM plan for every decode bucket and weight shape (before capture)."""
         m = self.model
+        if not self._paged_attn:
+            return                # layer-list models: heuristic plans (their projections are small next to the mixers)
         shapes = set()
         L = m.layers[0]
         for name in ("wqkv", "wqkv_f", "wo", "wgu", "wgu_f"):
@@ -350,7 +382,7 @@ class LLMEngine:
         return self.attn_worklist and bs >= self.ATTN_WL_MIN_BS
 
     def _attn_grid(self, bs: int) -> int:
-        return int(max(1, min(self.ATTN_PGRID, bs * self.model.nkv * self.max_splits)))
+        return int(max(1, min(self.ATTN_PGRID, bs * self._nkv * self.max_splits)))
 
     def _decode_splits(self, bs: int) -> int:
         if self.ATTN_DYNAMIC:
@@ -358,13 +390,13 @@ class LLMEngine:
         return self._splits_for(bs)
 
     def _split_len(self, total_ctx: int) -> int:
-        per = total_ctx * self.model.nkv / max(1, self.ATTN_TARGET_WGS)
+        per = total_ctx * self._nkv / max(1, self.ATTN_TARGET_WGS)
         return int(max(256, math.ceil(per / 256) * 256))
 
     def _splits_for(self, tiles: int) -> int:
         # measured on MI355X (scripts/microbench.py attn): split-K pays only while tiles x kv-heads
         # leaves CUs idle; at >= 256 work units one split is fastest.
-        return int(max(1, min(8, math.ceil(256 / max(1, tiles * self.model.nkv)))))
+        return int(max(1, min(8, math.ceil(256 / max(1, tiles * self._nkv)))))
 
     # ------------------------------------------------------------------ public API
     def encode(self, text: str) -> List[int]:
@@ -908,48 +940,7 @@ class LLMEngine:
             n = min(len(s.fill) - s.num_computed, budget)
             chunk.append((s, s.num_computed, s.num_computed + n))
             budget -= n
-        ids, pos, slots, qstart, qlen, ctx, last = [], [], [], [], [], [], []
-        G = self.model.nq // self.model.nkv
-        flash = self.on_gpu and ops.flash_supported(self.model.d, G, self.max_blocks)
-        tiler = ops.flash_tiles if flash else ops.build_tiles
-        tseq, ttok = [], []
-        t = 0
-        for i, (s, a, b) in enumerate(chunk):
-            ids.extend(s.fill[a:b])
-            pos.extend(range(a, b))
-            slots.extend(self.bm.slots(s.id, a, b))
-            qstart.append(t)
-            qlen.append(b - a)
-            ctx.append(b)
-            t += b - a
-            last.append(t - 1)
-            ts, tt = tiler([b - a], G)
-            tseq.extend([i] * len(ts))
-            ttok.extend(tt)
-        nb = max((ctx_i + BS - 1) // BS for ctx_i in ctx)
-        rows = np.fromiter((s.row for s, _, _ in chunk), dtype=np.int64, count=len(chunk))
-        bt = self.bt_host[rows, :nb]
-        dev = self.device
-        splits = self._splits_for(len(tseq))
-        if self.on_gpu:
-            # one pinned staging buffer, one async H2D copy: the host builds this chunk while the
-            # GPU still runs the previous one (per-tensor torch.tensor(..., device) copies sync)
-            (slots_d, qstart_d, qlen_d, ctx_d, tseq_d, ttok_d, last_d, ids_d, pos_d, bt_d) = self._stage_i32(
-                [slots, qstart, qlen, ctx, tseq, ttok, last, ids, pos, bt])
-            last_d = last_d.to(torch.int64)
-            bt_d = bt_d.view(len(chunk), nb)
-        else:
-            T = lambda x, dt=torch.int32: torch.tensor(x, dtype=dt, device=dev)
-            slots_d, qstart_d, qlen_d, ctx_d, tseq_d, ttok_d = T(slots), T(qstart), T(qlen), T(ctx), T(tseq), T(ttok)
-            last_d, ids_d, pos_d, bt_d = T(last, torch.int64), T(ids), T(pos), torch.from_numpy(np.ascontiguousarray(bt))
-        meta = AttnMeta(slots=slots_d, block_tables=bt_d, qstart=qstart_d, qlen=qlen_d,
-                        ctx=ctx_d, tile_seq=tseq_d, tile_tok0=ttok_d, last_idx=last_d,
-                        splits=splits, xcd_remap=True, flash=flash, max_ctx=max(ctx))
-        hidden = self.model.hidden_states(ids_d, pos_d, meta, self.kv_caches)
-        if not self._collectives_ok():
-            # a one-shot all-reduce timed out on some rank: every rank re-runs the chunk on RCCL
-            # (same inputs, the K/V slot writes are idempotent)
-            hidden = self.model.hidden_states(ids_d, pos_d, meta, self.kv_caches)
+        hidden, t = self._forward_chunk(chunk)
         self.steps["prefill"] += 1
         self.steps["prefill_tokens"] += t
         done_seqs = [s for (s, a, b) in chunk if b == len(s.fill)]
@@ -977,6 +968,64 @@ class LLMEngine:
             ev.record()
             return done_seqs, (self._pf_tok, ev)
         return done_seqs, toks
+
+    def _forward_chunk(self, chunk: List[tuple], want: Optional[List[int]] = None) -> Tuple[torch.Tensor, int]:
+        """One packed forward over ``chunk`` = [(sequence, first position, end position)]: the
+        tokens ``fill[a:b]`` of every sequence, attending to what the cache and state slots already
+        hold.  Returns the final-normed hidden states of the packed rows ``want`` (default: each
+        sequence's last new token) and the number of tokens run.  Portions of prompts and single
+        tokens of running sequences may share a chunk."""
+        ids, pos, slots, qstart, qlen, ctx, last = [], [], [], [], [], [], []
+        if self._paged_attn:
+            G = self.model.nq // self.model.nkv
+            flash = self.on_gpu and ops.flash_supported(self.model.d, G, self.max_blocks)
+            tiler = ops.flash_tiles if flash else ops.build_tiles
+        else:                      # the model tiles its own mixers (AttnMeta.host_qlen)
+            G, flash, tiler = 1, False, None
+        tseq, ttok = [], []
+        t = 0
+        for i, (s, a, b) in enumerate(chunk):
+            ids.extend(s.fill[a:b])
+            pos.extend(range(a, b))
+            slots.extend(self.bm.slots(s.id, a, b))
+            qstart.append(t)
+            qlen.append(b - a)
+            ctx.append(b)
+            t += b - a
+            last.append(t - 1)
+            if tiler is not None:
+                ts, tt = tiler([b - a], G)
+                tseq.extend([i] * len(ts))
+                ttok.extend(tt)
+        if want is not None:
+            last = list(want)
+        nb = max((ctx_i + BS - 1) // BS for ctx_i in ctx)
+        rows = np.fromiter((s.row for s, _, _ in chunk), dtype=np.int64, count=len(chunk))
+        bt = self.bt_host[rows, :nb]
+        dev = self.device
+        splits = self._splits_for(max(1, len(tseq)))
+        if self.on_gpu:
+            # one pinned staging buffer, one async H2D copy: the host builds this chunk while the
+            # GPU still runs the previous one (per-tensor torch.tensor(..., device) copies sync)
+            (slots_d, qstart_d, qlen_d, ctx_d, tseq_d, ttok_d, last_d, ids_d, pos_d, bt_d, rows_d) = self._stage_i32(
+                [slots, qstart, qlen, ctx, tseq, ttok, last, ids, pos, bt, rows])
+            last_d = last_d.to(torch.int64)
+            bt_d = bt_d.view(len(chunk), nb)
+        else:
+            T = lambda x, dt=torch.int32: torch.tensor(x, dtype=dt, device=dev)
+            slots_d, qstart_d, qlen_d, ctx_d, tseq_d, ttok_d = T(slots), T(qstart), T(qlen), T(ctx), T(tseq), T(ttok)
+            last_d, ids_d, pos_d, bt_d = T(last, torch.int64), T(ids), T(pos), torch.from_numpy(np.ascontiguousarray(bt))
+            rows_d = T(rows.tolist())
+        meta = AttnMeta(slots=slots_d, block_tables=bt_d, qstart=qstart_d, qlen=qlen_d,
+                        ctx=ctx_d, tile_seq=tseq_d, tile_tok0=ttok_d, last_idx=last_d,
+                        splits=splits, xcd_remap=True, flash=flash, max_ctx=max(ctx), state_rows=rows_d,
+                        host_qlen=list(qlen))
+        hidden = self.model.hidden_states(ids_d, pos_d, meta, self.kv_caches)
+        if not self._collectives_ok():
+            # a one-shot all-reduce timed out on some rank: every rank re-runs the chunk on RCCL
+            # (same inputs, the K/V slot writes are idempotent)
+            hidden = self.model.hidden_states(ids_d, pos_d, meta, self.kv_caches)
+        return hidden, t
 
     def _small_h2d(self, a: np.ndarray) -> torch.Tensor:
         """A few KB of int32 to the device without a host stall: through a ring of 4 pinned slots
@@ -1079,7 +1128,7 @@ class LLMEngine:
             grid = self._attn_grid(bs)
             target = self.ATTN_ITEMS_PER_WG * grid
             items_t, items = self._items_bufs[p]
-            ops.decode_work_items(lens[order], self.model.nkv, self.max_splits, target,
+            ops.decode_work_items(lens[order], self._nkv, self.max_splits, target,
                                   min_chunk=self.ATTN_MIN_CHUNK, out=items, seq=rows[order], qstart=order)
             n_items = ops.work_items_len(items)
         h[o[4]:o[6] + R + 1] = 0
@@ -1597,7 +1646,7 @@ class LLMEngine:
                             last_idx=self.d_last[:bs], all_last=True, splits=self.max_splits, workspace=self.dec_ws,
                             items=self.items_dev, grid_items=self._attn_grid(bs))
         return AttnMeta(slots=self.d_slots[:bs], block_tables=self.bt_dev, qstart=self.d_qstart, qlen=self.d_qlen,
-                        ctx=self.d_ctx, tile_seq=self.d_tseq[:bs], tile_tok0=self.d_tok0[:bs],
+                        ctx=self.d_ctx, tile_seq=self.d_tseq[:bs], tile_tok0=self.d_tok0[:bs], state_rows=self.d_rows,
                         last_idx=self.d_last[:bs], all_last=True, splits=self._decode_splits(bs), workspace=self.dec_ws,
                         split_len=self.d_split if self.ATTN_DYNAMIC else None)
 
@@ -1619,6 +1668,9 @@ class LLMEngine:
         # embedding launch)
         hid = self.model.hidden_states(self.d_ids[:bs], self.d_pos[:bs], self._decode_meta(bs), self.kv_caches,
                                        scatter=(self.bt_dev, self.d_upd))
+        if self.d_logits is not None:      # forced-token replay: the step's logits stay on the device
+            lf = getattr(self.model, "logits_f32", None)
+            self.d_logits[:bs].copy_(lf(hid) if lf is not None else self.model.logits(hid).float())
         if self.fused_sampler:
             self.model.sample(hid, self.d_temp[:bs], self.d_topp[:bs], self.d_topk[:bs], self.d_seed,
                               self.d_out[:bs])
@@ -1634,6 +1686,7 @@ class LLMEngine:
         # (step I/O kernels) the warm-up's sampler would overwrite the previous step's tokens the
         # replay gathers its input ids from, so d_out is restored after it.
         saved = self.d_out.clone() if self._gio else None
+        staged = self._stage_padding(p) if self.recurrent else None
         s = torch.cuda.Stream(device=self.device)
         s.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(s):
@@ -1647,7 +1700,33 @@ class LLMEngine:
         with torch.cuda.graph(g, pool=self._graph_pool):
             self._decode_forward(bs, p)
         self._graphs[self._gkey(bs, p)] = g
+        if staged is not None:
+            self._unstage_padding(p, staged)
         return g
+
+    def _stage_padding(self, p: int):
+        """A model with recurrent state must not run a real step twice: the warm-up run of a graph
+        captured mid-serving would advance every row's state.  Swap an all-padding step (no row
+        has new tokens, every slot -1) into staging buffer ``p`` for the warm-up; the real step is
+        put back once the warm-up has finished reading it."""
+        o, mb = self._off, self.buckets[-1]
+        _, h, _ = self._dec_bufs[p]
+        keep = h.copy()
+        dev_keep = self.dec_dev.clone()
+        h[:] = 0
+        h[o[2]:o[3]] = -1
+        h[o[3]:o[4]] = self.R
+        h[o[9]:o[9] + mb] = -1
+        if not self._gio:
+            self.dec_dev.copy_(self._dec_bufs[p][0])
+        return keep, dev_keep
+
+    def _unstage_padding(self, p: int, staged) -> None:
+        torch.cuda.synchronize(self.device)
+        keep, dev_keep = staged
+        self._dec_bufs[p][1][:] = keep
+        if not self._gio:
+            self.dec_dev.copy_(dev_keep)
 
     def capture_all(self, max_bs: Optional[int] = None) -> None:
         """Pre-capture decode graphs for every bucket up to ``max_bs`` (largest first)."""
@@ -1671,6 +1750,100 @@ class LLMEngine:
                 if self._gkey(b, p) not in self._graphs:
                     self._capture(b, p)
         torch.cuda.synchronize(self.device)
+
+    # ------------------------------------------------------------------ forced-token steps
+    def feed(self, entries: Sequence[Tuple[object, Sequence[int], Sequence[int]]],
+             end: Sequence[object] = ()) -> torch.Tensor:
+        """One engine step over GIVEN tokens (replaying a recorded schedule, scoring a text): nothing
+        is sampled.  ``entries`` = [(key, tokens, want)]: the next tokens of request ``key`` (admitted
+        at its first entry: a batch row / state slot and paged blocks, as any request) and the
+        places among them whose logits are wanted.  All entries run as ONE batch through the same
+        paths as generation: a step of single tokens of running requests is a decode step (graph
+        replay where decode uses graphs), anything else a packed chunk (``_forward_chunk``).
+        ``end``: requests that are finished after this step; their row and blocks are released.
+        Returns f32 logits [wanted, vocab] on the host, in entry and ``want`` order."""
+        with self._lock:
+            return self._feed(entries, end)
+
+    def _feed(self, entries, end) -> torch.Tensor:
+        seqs: List[_Seq] = []
+        now = time.perf_counter()
+        for key, toks, _ in entries:
+            toks = [int(t) for t in toks]
+            if not toks:
+                raise ValueError("an entry needs at least one token")
+            s = self._streams.get(key)
+            if s is None:
+                if not self._free_rows:
+                    raise RuntimeError("no free batch row / state slot for a new request")
+                s = _Seq(next(self._ids), toks, SamplingParams(temperature=0.0, max_new_tokens=1 << 30), now)
+                table, _ = self.bm.allocate(s.id, s.prompt)
+                if not table:
+                    raise RuntimeError("paged pool exhausted")
+                s.fill = s.prompt
+                s.row = self._free_rows.pop()
+                s.admitted = now
+                self._set_row_blocks(s)
+                self._streams[key] = s
+            else:
+                if s.length + len(toks) > self.max_model_len:
+                    raise RuntimeError("request longer than max_model_len")
+                for t in toks:
+                    slot = self.bm.append_token(s.id, t)
+                    if slot < 0:
+                        raise RuntimeError("paged pool exhausted")
+                    s.prompt.append(t)
+                    if slot % BS == 0:
+                        nblk = (len(s.prompt) + BS - 1) // BS
+                        self.bt_host[s.row, nblk - 1] = slot // BS
+                        self._bt_hw = max(self._bt_hw, nblk)
+                        self._bt_dirty = True      # the next decode step copies the table (_sync_bt)
+                        self._mark_bt_row(s.row)
+            seqs.append(s)
+        n_want = sum(len(w) for _, _, w in entries)
+        decode = all(len(t) == 1 and s.num_computed > 0 for s, (_, t, _) in zip(seqs, entries))
+        if decode:
+            if self.d_logits is None:
+                self.d_logits = torch.zeros((self.buckets[-1], self.cfg.vocab), dtype=torch.float32, device=self.device)
+                self._graphs.clear()        # graphs captured before did not keep the logits
+            B = len(seqs)
+            lens = np.fromiter((s.length for s in seqs), dtype=np.int64, count=B)
+            last = np.fromiter((s.prompt[-1] for s in seqs), dtype=np.int64, count=B)
+            bs = self._prep_decode(seqs, lens, last, 0)
+            if self.use_graphs:
+                self._replay(bs, 0)
+            else:
+                self._decode_forward(bs, 0)
+            self.steps["decode"] += 1
+            self.steps["decode_tokens"] += B
+            rows = [i for i, (_, _, w) in enumerate(entries) for _ in w]
+            out = self.d_logits[:B].cpu()[rows] if rows else torch.empty((0, self.cfg.vocab))
+        else:
+            chunk, want, t0 = [], [], 0
+            for s, (_, toks, w) in zip(seqs, entries):
+                chunk.append((s, s.num_computed, s.length))
+                want.extend(t0 + int(j) for j in w)
+                t0 += len(toks)
+            with ops.gemm.workspace_owner(self._ws_owner):
+                hidden, t = self._forward_chunk(chunk, want=want if want else [0])
+            self.steps["prefill"] += 1
+            self.steps["prefill_tokens"] += t
+            if want:
+                lf = getattr(self.model, "logits_f32", None)
+                out = (lf(hidden) if lf is not None else self.model.logits(hidden).float()).cpu()
+            else:
+                out = torch.empty((0, self.cfg.vocab))
+                if self.on_gpu:
+                    torch.cuda.current_stream(self.device).synchronize()
+        for s in seqs:
+            s.num_computed = s.length
+            self.bm.commit(s.id, s.length)
+        for key in end:
+            s = self._streams.pop(key, None)
+            if s is not None:
+                self._release(s)
+        assert out.shape[0] == n_want
+        return out
 
     # ------------------------------------------------------------------ outputs
     def _finalize_text(self, s: _Seq) -> str:

@@ -7,8 +7,10 @@ src/devices/orin_api.py:18).
 """
 from __future__ import annotations
 
+import json
+import os
 from dataclasses import dataclass, field, replace
-from typing import Dict, Optional
+from typing import Dict, Optional, Tuple, Union
 
 
 @dataclass(frozen=True)
@@ -81,3 +83,158 @@ def get_model_config(name: str, **overrides) -> ModelConfig:
         raise KeyError(f"unknown model {name!r}; known: {sorted(MODELS)}")
     cfg = MODELS[key]
     return replace(cfg, **overrides) if overrides else cfg
+
+
+# ----------------------------------------------------------------------------- layer-list designs
+#
+# A hybrid design is a list of layers, each with a token mixer (state-space scan, retention, latent
+# attention) and an optional feed-forward; every size and constant comes from the model folder's
+# config.json.  ``family`` picks the model class (models.registry).
+
+@dataclass(frozen=True)
+class RopeSpec:
+    dims: int
+    base: float
+
+
+@dataclass(frozen=True)
+class MixerSpec:
+    """One token mixer.  ``kind``: ``mamba1`` (inner, state, dt_rank, conv), ``retention`` (heads,
+    dim, vdim, decay per head, rot) or ``latent_attention`` (heads, dim, rot_dim, vdim, kv_rank,
+    q_rank, scale, rot)."""
+    kind: str
+    inner: int = 0
+    state: int = 0
+    dt_rank: int = 0
+    conv: int = 0
+    heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    decay: Tuple[float, ...] = ()
+    rot: Optional[RopeSpec] = None
+    rot_dim: int = 0
+    kv_rank: int = 0
+    q_rank: int = 0
+    scale: float = 1.0
+
+    @property
+    def recurrent(self) -> bool:
+        return self.kind in ("mamba1", "retention")
+
+
+@dataclass(frozen=True)
+class MoESpec:
+    """Routed experts (``ff`` wide, ``top`` of ``experts`` per token, weights times ``scale``) and an
+    optional shared expert (``shared_ff`` > 0) that every token runs."""
+    experts: int
+    top: int
+    scale: float
+    ff: int
+    shared_ff: int = 0
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    mixer: MixerSpec
+    mlp: Optional[MoESpec] = None
+
+
+@dataclass(frozen=True)
+class HybridConfig:
+    name: str
+    family: str
+    hidden: int
+    vocab: int
+    layers: Tuple[LayerSpec, ...]
+    rms_eps: float = 1e-6
+    logit_scale: float = 1.0
+    max_position: int = 1 << 20       # the design has no position limit; the engine's max_model_len bounds it
+    bos_id: int = 1
+    eos_id: int = 2
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(L.mlp is not None for L in self.layers)
+
+    def num_params(self) -> int:
+        H, n = self.hidden, 2 * self.vocab * self.hidden + self.hidden
+        for L in self.layers:
+            m = L.mixer
+            if m.kind == "mamba1":
+                n += 2 * m.inner * H + m.inner * (m.conv + 1) + (m.dt_rank + 2 * m.state) * m.inner
+                n += m.inner * (m.dt_rank + 1) + m.inner * m.state + m.inner + H * m.inner
+            elif m.kind == "retention":
+                n += 2 * m.heads * m.dim * H + 2 * m.heads * m.vdim * H + H * m.heads * m.vdim
+            else:
+                n += m.q_rank * (H + 1) + m.heads * (m.dim + m.rot_dim) * m.q_rank + (m.kv_rank + m.rot_dim) * H
+                n += m.kv_rank + m.heads * (m.dim + m.vdim) * m.kv_rank + H * m.heads * m.vdim
+            n += H
+            if L.mlp is not None:
+                f = L.mlp
+                n += H + f.experts * (H + 2 * f.ff * H) + 2 * f.shared_ff * H
+        return n
+
+
+def _rope(d: Optional[dict]) -> Optional[RopeSpec]:
+    return RopeSpec(int(d["dims"]), float(d["base"])) if d else None
+
+
+def filevik_config(raw: dict, name: str = "filevik") -> HybridConfig:
+    """A Filevik config.json: ``layers`` (type, mixer sizes, mlp or null), ``norm.eps``,
+    ``logit_scale``, ``vocab``, ``width``."""
+    layers = []
+    for L in raw["layers"]:
+        m, kind = L["mixer"], L["type"]
+        if kind == "mamba1":
+            mix = MixerSpec(kind, inner=int(m["inner"]), state=int(m["state"]), dt_rank=int(m["dt_rank"]),
+                            conv=int(m["conv"]))
+        elif kind == "retention":
+            mix = MixerSpec(kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                            decay=tuple(float(x) for x in m["decay"]), rot=_rope(m.get("rot")))
+        elif kind == "latent_attention":
+            mix = MixerSpec(kind, heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]),
+                            vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]),
+                            scale=float(m["scale"]), rot=_rope(m.get("rot")))
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        f = L.get("mlp")
+        mlp = None
+        if f:
+            if f.get("kind", "moe") != "moe":
+                raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+            sh = f.get("shared")
+            mlp = MoESpec(int(f["router"]["experts"]), int(f["router"]["top"]), float(f["router"].get("scale", 1.0)),
+                          int(f["expert"]["ff"]), int(sh["ff"]) if sh else 0)
+        layers.append(LayerSpec(mix, mlp))
+    return HybridConfig(name, "filevik", int(raw["width"]), int(raw["vocab"]), tuple(layers),
+                        rms_eps=float(raw["norm"]["eps"]), logit_scale=float(raw.get("logit_scale", 1.0)))
+
+
+# config.json "architecture" -> parser of that design's keys
+ARCHITECTURES = {"Filevik": filevik_config}
+
+AnyConfig = Union[ModelConfig, HybridConfig]
+
+
+def config_from_dir(path: str) -> AnyConfig:
+    """The configuration of a model folder (config.json + model.safetensors): the parser is chosen
+    by the file's ``architecture``."""
+    with open(os.path.join(path, "config.json")) as f:
+        raw = json.load(f)
+    arch = raw.get("architecture")
+    if arch not in ARCHITECTURES:
+        raise KeyError(f"unknown architecture {arch!r}; known: {sorted(ARCHITECTURES)}")
+    return ARCHITECTURES[arch](raw, name=os.path.basename(os.path.normpath(path)) or arch.lower())
+
+
+def resolve_config(model: Union[str, AnyConfig]) -> AnyConfig:
+    """A registry name, a model folder, or a config object -> config."""
+    if not isinstance(model, str):
+        return model
+    if os.path.isdir(model) and os.path.exists(os.path.join(model, "config.json")):
+        return config_from_dir(model)
+    return get_model_config(model)

@@ -62,6 +62,28 @@ class AttnMeta:
     flash: bool = False                        # prefill: tile_seq/tile_tok0 are 128-row flash tiles
     max_ctx: int = 0                           # prefill: longest context (host-known; flash split-KV choice)
     all_last: bool = False                     # decode: every row is its sequence's last token (no gather)
+    state_rows: Optional[torch.Tensor] = None  # [S] recurrent-state slot of each sequence (layer-list models)
+    host_qlen: Optional[List[int]] = None      # prefill: new tokens per sequence, on the host
+    _lat: Optional[Dict[int, Tuple[torch.Tensor, torch.Tensor]]] = None
+
+    def latent_tiles(self, heads: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(sequence, first token) entries of the latent attention kernel for ``heads`` heads: an
+        entry covers max(1, 16 // heads) tokens.  Decode steps (one token per sequence) use the
+        step's own tile table; prefill builds one per head count from ``host_qlen``."""
+        if self.host_qlen is None:
+            return self.tile_seq, self.tile_tok0
+        if self._lat is None:
+            self._lat = {}
+        tpe = max(1, 16 // heads)
+        if tpe not in self._lat:
+            ts, tt = [], []
+            for i, n in enumerate(self.host_qlen):
+                for t0 in range(0, int(n), tpe):
+                    ts.append(i)
+                    tt.append(t0)
+            self._lat[tpe] = (torch.tensor(ts, dtype=torch.int32, device=device),
+                              torch.tensor(tt, dtype=torch.int32, device=device))
+        return self._lat[tpe]
 
 
 def qk_dim_order(d: int) -> torch.Tensor:

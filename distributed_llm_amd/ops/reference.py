@@ -360,3 +360,193 @@ def embedding(ids, table, lo=0):
     local = ids.reshape(-1).long() - lo
     ok = (local >= 0) & (local < table.shape[0])
     return table[local.clamp(0, table.shape[0] - 1)] * ok.unsqueeze(-1).to(table.dtype)
+
+
+# ----------------------------------------------------------------------------- sequence mixers
+#
+# Shared conventions of the recurrent / latent mixers (csrc/kernels/seqmix.hip, latent.hip): a step
+# is a packed batch of S sequences; sequence s brings tokens [qstart[s], qstart[s] + qlen[s]) at
+# positions [ctx[s] - qlen[s], ctx[s]) and keeps its recurrent state in slot rows[s].  A sequence
+# whose first new position is 0 starts from a zero state whatever its slot holds.
+
+def _seq_meta(qstart, qlen, ctx, rows):
+    qs, ql, cx = qstart.tolist(), qlen.tolist(), ctx.tolist()
+    rw = rows.tolist() if rows is not None else list(range(len(qs)))
+    return [(qs[i], ql[i], cx[i], rw[i]) for i in range(len(qs)) if ql[i] > 0]
+
+
+def rms_rows(x, w, eps, out_dtype=None):
+    xf = x.float()
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    if w is not None:
+        y = y * w.float()
+    return y.to(out_dtype or x.dtype)
+
+
+def norm_resadd(y, w, eps, x, x_lp=None):
+    """x (f32 residual stream, in place) += rmsnorm(y) * w; ``x_lp`` receives x rounded to its dtype."""
+    x += rms_rows(y, w, eps, torch.float32)
+    if x_lp is not None:
+        x_lp.copy_(x)
+    return x
+
+
+def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows):
+    """y[t, c] = silu(b[c] + sum_k w[c, k] u[t - K + 1 + k, c]) over each sequence's inputs u (the
+    slot's last K - 1 inputs before its new tokens, zeros before position 0).  x [T, >= C] (first C
+    columns), conv_state [slots, K - 1, C].  The state is NOT updated (selective_scan does)."""
+    C, K = w.shape
+    y = torch.zeros((x.shape[0], C), dtype=x.dtype, device=x.device)
+    wf = w.float()
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        hist = conv_state[row].float() if cx - n > 0 else torch.zeros((K - 1, C), dtype=torch.float32, device=x.device)
+        u = torch.cat([hist, x[q0:q0 + n, :C].float()], 0)
+        acc = b.float()[None, :].expand(n, C).clone()
+        for k in range(K):
+            acc += u[k:k + n] * wf[:, k][None, :]
+        y[q0:q0 + n] = torch.nn.functional.silu(acc).to(x.dtype)
+    return y
+
+
+def selective_scan(xc, dt_raw, dt_bias, A, dbc, dt_rank, D, xz, ssm_state, conv_state, qstart, qlen, ctx, rows):
+    """Mamba-1 recurrence with the output gate.  xc [T, C] (convolved, activated), dt_raw [T, C],
+    A [C, N] f32 (negative), dbc [T, dt_rank + 2N] (B at dt_rank, C at dt_rank + N), xz [T, 2C]
+    (x | z: z gates, x refills the convolution state).  Per channel: S <- exp(dt A) S + dt x B,
+    y = S . C + D x, out = y silu(z).  Updates ssm_state [slots, C, N] f32 and conv_state."""
+    C, N = A.shape
+    Km1 = conv_state.shape[1]
+    out = torch.zeros_like(xc)
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        S = ssm_state[row].clone() if cx - n > 0 else torch.zeros((C, N), dtype=torch.float32, device=xc.device)
+        dt = torch.nn.functional.softplus(dt_raw[q0:q0 + n].float() + dt_bias.float()[None, :], threshold=30.0)
+        xs = xc[q0:q0 + n].float()
+        Bm = dbc[q0:q0 + n, dt_rank:dt_rank + N].float()
+        Cm = dbc[q0:q0 + n, dt_rank + N:dt_rank + 2 * N].float()
+        ys = torch.empty((n, C), dtype=torch.float32, device=xc.device)
+        for t in range(n):
+            S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * xs[t])[:, None] * Bm[t][None, :]
+            ys[t] = S @ Cm[t] + D.float() * xs[t]
+        z = xz[q0:q0 + n, C:2 * C].float()
+        out[q0:q0 + n] = (ys * torch.nn.functional.silu(z)).to(xc.dtype)
+        ssm_state[row] = S
+        if Km1 > 0:
+            hist = conv_state[row].float() if cx - n > 0 else torch.zeros((Km1, C), dtype=torch.float32, device=xc.device)
+            u = torch.cat([hist, xz[q0:q0 + n, :C].float()], 0)
+            conv_state[row] = u[-Km1:].to(conv_state.dtype)
+    return out
+
+
+def _rot_table(cos_sin, pos, half):
+    """cos, sin [n, half] of positions ``pos`` from a [max_pos, 2 * half] table (cos | sin)."""
+    t = cos_sin.index_select(0, pos.long())
+    return t[:, :half], t[:, half:2 * half]
+
+
+def retention(qkvg, heads, dim, vdim, cos_sin, rot_dims, decay, state, eps, positions, qstart, qlen, ctx, rows):
+    """Decayed linear attention with rotate-half positions on the first ``rot_dims`` dims of q and k,
+    k scaled by dim^-1/2, unit-RMS heads and a SiLU gate.  qkvg [T, 2 heads dim + 2 heads vdim]
+    (q | k | v | gate); state [slots, heads, dim, vdim] f32; returns [T, heads * vdim]."""
+    T = qkvg.shape[0]
+    H, d, dv = heads, dim, vdim
+    out = torch.zeros((T, H * dv), dtype=qkvg.dtype, device=qkvg.device)
+    half = rot_dims // 2
+    dec = decay.float()
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        blk = qkvg[q0:q0 + n].float()
+        q = blk[:, :H * d].reshape(n, H, d).clone()
+        k = blk[:, H * d:2 * H * d].reshape(n, H, d).clone()
+        v = blk[:, 2 * H * d:2 * H * d + H * dv].reshape(n, H, dv)
+        g = blk[:, 2 * H * d + H * dv:]
+        if half > 0:
+            c, s = _rot_table(cos_sin, positions[q0:q0 + n], half)
+            c, s = c[:, None, :], s[:, None, :]
+            for t_ in (q, k):
+                u, w_ = t_[..., :half].clone(), t_[..., half:2 * half].clone()
+                t_[..., :half] = u * c - w_ * s
+                t_[..., half:2 * half] = w_ * c + u * s
+        k = k * (d ** -0.5)
+        S = state[row].clone() if cx - n > 0 else torch.zeros((H, d, dv), dtype=torch.float32, device=qkvg.device)
+        o = torch.empty((n, H, dv), dtype=torch.float32, device=qkvg.device)
+        for t in range(n):
+            S = dec[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[row] = S
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        out[q0:q0 + n] = (o.reshape(n, H * dv) * torch.nn.functional.silu(g)).to(qkvg.dtype)
+    return out
+
+
+def _rope_interleaved(x, c, s):
+    u, w_ = x[..., 0::2], x[..., 1::2]
+    out = torch.empty_like(x)
+    out[..., 0::2] = u * c - w_ * s
+    out[..., 1::2] = w_ * c + u * s
+    return out
+
+
+def latent_kv_write(ckv, rank, norm_w, eps, positions, cos_sin, slots, cache):
+    """cache[slot] = [rmsnorm(ckv[:, :rank]) * norm_w | interleaved-rotated ckv[:, rank:]]."""
+    dr = ckv.shape[1] - rank
+    c = rms_rows(ckv[:, :rank], norm_w, eps, torch.float32)
+    cs, sn = _rot_table(cos_sin, positions, dr // 2)
+    kr = _rope_interleaved(ckv[:, rank:].float(), cs, sn)
+    ok = slots >= 0
+    cache.view(-1, cache.shape[-1])[slots[ok].long()] = torch.cat([c, kr], 1)[ok].to(cache.dtype)
+
+
+def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx, scale):
+    """Causal softmax attention over a shared latent: row (t, h) scores key j as
+    (qa[h, t] . c_j + rot(q[t, h, dim:]) . kr_j) * scale and returns sum_j p_j c_j.
+    qa [heads, T, rank], q [T, heads * (dim + rot_dim)], cache [blocks, 16, rank + rot_dim]."""
+    Hh, T, r = qa.shape
+    out = torch.zeros((Hh, T, r), dtype=qa.dtype, device=qa.device)
+    flat = cache.view(-1, cache.shape[-1])
+    qs, ql, cx = qstart.tolist(), qlen.tolist(), ctx.tolist()
+    for s in range(len(qs)):
+        n = ql[s]
+        if n <= 0:
+            continue
+        q0, L = qs[s], cx[s]
+        nb = (L + BS - 1) // BS
+        idx = (block_tables[s, :nb].long()[:, None] * BS + torch.arange(BS, device=cache.device)[None, :]).reshape(-1)[:L]
+        kv = flat[idx].float()
+        cs, sn = _rot_table(cos_sin, positions[q0:q0 + n], rot_dim // 2)
+        qr = q[q0:q0 + n].float().reshape(n, Hh, dim + rot_dim)[..., dim:]
+        qr = _rope_interleaved(qr, cs[:, None, :], sn[:, None, :])
+        sc = (torch.einsum("htr,jr->htj", qa[:, q0:q0 + n].float(), kv[:, :r]) +
+              torch.einsum("thr,jr->htj", qr, kv[:, r:])) * scale
+        pos = positions[q0:q0 + n].long()
+        mask = torch.arange(L, device=cache.device)[None, :] <= pos[:, None]
+        sc = sc.masked_fill(~mask[None], float("-inf"))
+        p = torch.softmax(sc, -1)
+        out[:, q0:q0 + n] = torch.einsum("htj,jr->htr", p, kv[:, :r]).to(qa.dtype)
+    return out
+
+
+def relu2_scale(x, gate=None, ff=0):
+    """relu(x)^2, optionally times gate[t, column // ff] (dense routed experts: a token's weight of
+    the column's expert, zero for experts it does not use)."""
+    y = torch.relu(x.float()) ** 2
+    if gate is not None:
+        y = y * gate.float().repeat_interleave(ff, dim=1)
+    return y.to(x.dtype)
+
+
+def moe_ffn_relu2(x, ids, wts, w1, w2):
+    """sum_j wts[t, j] * relu(x w1_e^T)^2 w2_e^T with e = ids[t, j] (w1 [E, I, H], w2 [E, H, I])."""
+    T, H = x.shape
+    out = torch.zeros((T, H), dtype=torch.float32, device=x.device)
+    xf = x.float()
+    for j in range(ids.shape[1]):
+        for e in ids[:, j].unique().tolist():
+            sel = (ids[:, j] == e).nonzero().flatten()
+            act = (torch.relu(xf[sel] @ w1[e].float().t()) ** 2).to(x.dtype).float()
+            out[sel] += wts[sel, j:j + 1].float() * (act @ w2[e].float().t())
+    return out.to(x.dtype)
+
+
+def dense_gate(ids, wts, E):
+    """[T, E] f32: wts scattered to their experts' columns, zero elsewhere."""
+    g = torch.zeros((ids.shape[0], E), dtype=torch.float32, device=ids.device)
+    g.scatter_(1, ids.long(), wts.float())
+    return g

@@ -1,0 +1,131 @@
+"""Sequence-mixer ops beside softmax attention: short causal convolution, selective scan, decayed
+linear attention (retention), latent attention over a shared compressed key/value, the f32
+residual update, squared-ReLU experts (csrc/kernels/seqmix.hip, latent.hip, moe.hip).
+
+Same dispatch rule as the rest of the op library: GPU tensors run the HIP kernel (or raise when the
+extension is missing), CPU tensors the torch reference.  Every kernel takes bf16 or f32 activations
+(the model's dtype) and computes scores, states, norms and gates in f32.
+
+A step is a packed batch of S sequences: sequence s brings tokens [qstart[s], qstart[s] + qlen[s])
+at positions [ctx[s] - qlen[s], ctx[s]) and keeps its recurrent state in slot ``rows[s]``.  A
+sequence whose first new position is 0 starts from a zero state, so a re-used slot needs no reset.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _native, reference as ref
+
+LAT_ROWS = 16      # (token, head) rows per workgroup of the latent attention kernel; a tile entry
+                   # (sequence, first token) covers max(1, 16 // heads) tokens (AttnMeta.latent_tiles)
+
+
+def rms_rows(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype=None) -> torch.Tensor:
+    """Row-wise x / sqrt(mean(x^2) + eps) (* w) for any row length; x may be a column slice."""
+    ext = _native(x)
+    if ext is None:
+        return ref.rms_rows(x, w, eps, out_dtype)
+    y = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    ext.rms_rows(x, w, y, float(eps))
+    return y
+
+
+def norm_resadd(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor,
+                x_lp: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Residual update in f32: ``x += rmsnorm(y) * w`` in place (x f32 [T, H]); ``x_lp`` (the model
+    dtype) receives the rounded stream for the next projections, in the same launch."""
+    ext = _native(y)
+    if ext is None:
+        return ref.norm_resadd(y, w, eps, x, x_lp)
+    ext.norm_resadd(y, w, float(eps), x, x_lp)
+    return x
+
+
+def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows) -> torch.Tensor:
+    ext = _native(x)
+    if ext is None:
+        return ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows)
+    # rows of no sequence (graph padding) stay zero, never stale memory
+    y = torch.zeros((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
+    ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y)
+    return y
+
+
+def selective_scan(xc, dt_raw, dt_bias, A, dbc, dt_rank, D, xz, ssm_state, conv_state, qstart, qlen, ctx,
+                   rows) -> torch.Tensor:
+    ext = _native(xc)
+    if ext is None:
+        return ref.selective_scan(xc, dt_raw, dt_bias, A, dbc, dt_rank, D, xz, ssm_state, conv_state, qstart, qlen,
+                                  ctx, rows)
+    out = torch.zeros_like(xc)
+    ext.selective_scan(xc, dt_raw, dt_bias, A, dbc, int(dt_rank), D, xz, ssm_state, conv_state, qstart, qlen, ctx,
+                       rows, out)
+    return out
+
+
+def retention(qkvg, heads, dim, vdim, cos_sin, rot_dims, decay, state, eps, positions, qstart, qlen, ctx,
+              rows) -> torch.Tensor:
+    ext = _native(qkvg)
+    if ext is None:
+        return ref.retention(qkvg, heads, dim, vdim, cos_sin, rot_dims, decay, state, eps, positions, qstart, qlen,
+                             ctx, rows)
+    out = torch.zeros((qkvg.shape[0], heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    ext.retention(qkvg, int(heads), int(dim), int(vdim), cos_sin, int(rot_dims), decay, state, float(eps), positions,
+                  qstart, qlen, ctx, rows, out)
+    return out
+
+
+def latent_kv_write(ckv, rank, norm_w, eps, positions, cos_sin, slots, cache) -> None:
+    ext = _native(ckv)
+    if ext is None:
+        return ref.latent_kv_write(ckv, rank, norm_w, eps, positions, cos_sin, slots, cache)
+    ext.latent_kv_write(ckv, int(rank), norm_w, float(eps), positions, cos_sin, slots, cache)
+
+
+def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx, tile_seq,
+                     tile_tok0, scale) -> torch.Tensor:
+    ext = _native(qa)
+    if ext is None:
+        return ref.latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
+                                    scale)
+    out = torch.zeros_like(qa)
+    ext.latent_attention(qa, q, int(dim), int(rot_dim), positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
+                         tile_seq, tile_tok0, float(scale), out)
+    return out
+
+
+def relu2_scale(x: torch.Tensor, gate: Optional[torch.Tensor] = None, ff: int = 0) -> torch.Tensor:
+    ext = _native(x)
+    if ext is None:
+        return ref.relu2_scale(x, gate, ff)
+    y = torch.empty_like(x)
+    ext.relu2_scale(x, gate, int(ff), y)
+    return y
+
+
+def moe_ffn_relu2(x, ids, wts, w1, w2) -> torch.Tensor:
+    """Top-k experts with a squared-ReLU activation and no gate projection on the grouped MFMA
+    kernels of the SwiGLU experts (csrc/kernels/moe.hip, activation mode 1)."""
+    ext = _native(x)
+    if ext is None:
+        return ref.moe_ffn_relu2(x, ids, wts, w1, w2)
+    out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    ext.moe_ffn(x, ids.to(torch.int32).contiguous(), wts.float().contiguous(), w1, w2, out, 1)
+    return out
+
+
+def moe_ffn_relu2_ok(x: torch.Tensor, w1: torch.Tensor) -> bool:
+    """The grouped kernels need bf16 and 32-aligned widths; other shapes run the dense form."""
+    return (x.dtype == torch.bfloat16 and x.shape[1] % 32 == 0 and w1.shape[1] % 32 == 0 and w1.shape[0] <= 64
+            and x.stride(1) == 1 and x.stride(0) % 8 == 0)
+
+
+def dense_gate(ids, wts, E) -> torch.Tensor:
+    ext = _native(ids)
+    if ext is None:
+        return ref.dense_gate(ids, wts, E)
+    g = torch.zeros((ids.shape[0], E), dtype=torch.float32, device=ids.device)   # fill kernel (graph-safe)
+    ext.dense_gate(ids.to(torch.int32).contiguous(), wts.float().contiguous(), g)
+    return g
