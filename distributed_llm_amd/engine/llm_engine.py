@@ -1817,7 +1817,14 @@ class LLMEngine:
             self.steps["decode"] += 1
             self.steps["decode_tokens"] += B
             rows = [i for i, (_, _, w) in enumerate(entries) for _ in w]
-            out = self.d_logits[:B].cpu()[rows] if rows else torch.empty((0, self.cfg.vocab))
+            # the step must finish before the next one restages its pinned inputs (generation reads
+            # the step's tokens back at this point)
+            if rows:
+                out = self.d_logits[:B].cpu()[rows]
+            else:
+                out = torch.empty((0, self.cfg.vocab))
+                if self.on_gpu:
+                    torch.cuda.current_stream(self.device).synchronize()
         else:
             chunk, want, t0 = [], [], 0
             for s, (_, toks, w) in zip(seqs, entries):
