@@ -105,6 +105,12 @@ def parse():
                          "for token-exact cross-topology checks")
     ap.add_argument("--dump-responses", default=None,
                     help="rank 0 writes every timed turn's (conversation, turn, tier, response text) as JSON here")
+    ap.add_argument("--arch-bench", action="store_true",
+                    help="instead of the routing workload: a layer-list (Filevik) model beside the closest "
+                         "Llama-family model at equal size, prefill / decode throughput and mixer-kernel rooflines "
+                         "(prints its own JSON object)")
+    ap.add_argument("--arch-size", default="s", choices=["s", "m"])
+    ap.add_argument("--arch-kernels-only", action="store_true")
     ap.add_argument("--trace", default=None,
                     help="write a Chrome trace (router/pool/engine spans, GPU decode time) to this path; "
                          "'{rank}' is replaced by the rank")
@@ -479,6 +485,10 @@ def engine_time_split(st0, st1, window_s: float) -> dict:
 
 def main() -> int:
     a = parse()
+    if a.arch_bench:
+        from distributed_llm_amd.bench import arch_bench
+        arch_bench.run(a.arch_size, kernels_only=a.arch_kernels_only)
+        return 0
     if os.environ.get("DLLM_STACK_DUMP_S"):   # diagnostics: every thread's stack after S seconds (hang hunting)
         import faulthandler
         faulthandler.dump_traceback_later(float(os.environ["DLLM_STACK_DUMP_S"]), exit=False)

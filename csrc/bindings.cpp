@@ -58,6 +58,9 @@ int dllm_selective_scan(const void*, const void*, int, const float*, const float
 long dllm_retention_lds(int, int);
 int dllm_retention(const void*, long, int, int, int, int, const float*, int, int, const float*, float*, float,
                    const int*, const int*, const int*, const int*, void*, int, hipStream_t);
+long dllm_retention_chunk_lds(int);
+int dllm_retention_chunked(const void*, long, int, int, int, int, const float*, int, int, const float*, float*, float,
+                           const int*, const int*, const int*, const int*, float*, void*, int, long, hipStream_t);
 int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
 int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
 int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
@@ -1391,7 +1394,8 @@ void selective_scan(torch::Tensor xc, torch::Tensor dt_raw, torch::Tensor dt_bia
 
 void retention(torch::Tensor qkvg, int64_t H, int64_t d, int64_t dv, torch::Tensor cos_sin, int64_t rot,
                torch::Tensor decay, torch::Tensor state, double eps, torch::Tensor pos, torch::Tensor qstart,
-               torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor out) {
+               torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor out,
+               c10::optional<torch::Tensor> raw) {
   const bool f = act_f32(qkvg, "qkvg");
   check_rows2d(qkvg, "qkvg");
   check_f32(cos_sin, "cos_sin");
@@ -1407,8 +1411,19 @@ void retention(torch::Tensor qkvg, int64_t H, int64_t d, int64_t dv, torch::Tens
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == qkvg.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
                   out.size(0) == T && out.size(1) == H * dv,
               "out [T, H dv]");
-  TORCH_CHECK(dllm_retention_lds((int)d, (int)dv) <= 150 * 1024, "dim x vdim state does not fit the LDS");
   auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  if (raw) {   // chunked form (prompt portions): f32 scratch [T, H, dv]
+    check_f32(*raw, "raw");
+    TORCH_CHECK(raw->numel() >= (int64_t)T * H * dv, "raw scratch [T, H, dv]");
+    TORCH_CHECK(dllm_retention_chunk_lds((int)d) <= 150 * 1024, "dim does not fit the LDS");
+    ok(dllm_retention_chunked(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, cos_sin.data_ptr<float>(),
+                              (int)cos_sin.size(1), (int)rot, decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps,
+                              m.qstart, m.qlen, m.ctx, m.rows, raw->data_ptr<float>(), out.data_ptr(), m.S, (long)T,
+                              stream()),
+       "retention (chunked)");
+    return;
+  }
+  TORCH_CHECK(dllm_retention_lds((int)d, (int)dv) <= 150 * 1024, "dim x vdim state does not fit the LDS");
   ok(dllm_retention(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, cos_sin.data_ptr<float>(),
                     (int)cos_sin.size(1), (int)rot, decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps, m.qstart,
                     m.qlen, m.ctx, m.rows, out.data_ptr(), m.S, stream()),
@@ -1502,7 +1517,9 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("norm_resadd", &norm_resadd);
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("selective_scan", &selective_scan);
-  m.def("retention", &retention);
+  m.def("retention", &retention, py::arg("qkvg"), py::arg("heads"), py::arg("dim"), py::arg("vdim"), py::arg("cos_sin"),
+        py::arg("rot"), py::arg("decay"), py::arg("state"), py::arg("eps"), py::arg("positions"), py::arg("qstart"),
+        py::arg("qlen"), py::arg("ctx"), py::arg("rows"), py::arg("out"), py::arg("raw") = py::none());
   m.def("relu2_scale", &relu2_scale);
   m.def("dense_gate", &dense_gate);
   m.def("latent_kv_write", &latent_kv_write);

@@ -10,6 +10,9 @@
 //   retention        decayed linear attention: one workgroup per (sequence, head), the [dim x vdim]
 //                    state in LDS, rotate-half positions applied while q / k are staged, unit-RMS
 //                    heads and the SiLU gate in the same launch
+//   retention_chunk  the same recurrence for prompt portions in its chunked form (32 tokens at a time:
+//                    scores inside the chunk + the carried state), one workgroup per (head, 32 value
+//                    columns, sequence); retention_finish norms and gates
 //   relu2_scale      relu(x)^2 (* a per-(token, expert) gate): squared-ReLU experts, dense form
 //   dense_gate       top-k (id, weight) pairs -> [T, E] gate matrix
 //
@@ -92,7 +95,15 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x,
 }
 
 // ---------------------------------------------------------------- selective scan
-// 16 lanes per channel; lane `sub` owns states sub, sub + 16, ... (NS of them).
+// 16 lanes per channel; lane `sub` owns states sub, sub + 16, ... (NS of them).  Tokens run in
+// groups of 16: the group's B / C rows are staged once per workgroup in LDS (every channel reads the
+// same rows), and lane `sub` of a channel prepares token `sub` of the group (softplus step, input,
+// gate) and finishes it (skip term, SiLU gate, store), so the serial part of a token is only the
+// state update itself: NS exponentials and multiply-adds, a 16-lane sum, two broadcasts.
+template <typename T> struct fastexp;
+template <> struct fastexp<u16> { static __device__ __forceinline__ float f(float x) { return __expf(x); } };
+template <> struct fastexp<float> { static __device__ __forceinline__ float f(float x) { return expf(x); } };
+
 template <typename T, int NS>
 __global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, const T* __restrict__ dt_raw,
                                                    const float* __restrict__ dt_bias, const float* __restrict__ A,
@@ -102,12 +113,16 @@ __global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, con
                                                    const int* __restrict__ qstart, const int* __restrict__ qlen,
                                                    const int* __restrict__ ctx, const int* __restrict__ rows,
                                                    T* __restrict__ out, int C, int N) {
+  __shared__ float bcs[16 * 256];       // [16 tokens][2N], N <= 128
   const int s = blockIdx.y;
   const int n = qlen[s];
-  if (n <= 0) return;
-  const int c = blockIdx.x * 16 + (threadIdx.x >> 4), sub = threadIdx.x & 15;
-  if (c >= C) return;   // the 16 lanes of a channel leave together
+  if (n <= 0) return;                   // the whole workgroup
+  const int tid = threadIdx.x, sub = tid & 15;
+  const int c0 = blockIdx.x * 16 + (tid >> 4);
+  const bool live = c0 < C;
+  const int c = live ? c0 : C - 1;      // idle channels shadow the last one and store nothing
   const int q0 = qstart[s], p0 = ctx[s] - n, row = rows[s];
+  const int N2 = 2 * N;
   float a[NS], S[NS];
   float* sp = ssm + ((long)row * C + c) * N;
 #pragma unroll
@@ -117,28 +132,39 @@ __global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, con
     S[i] = (nn < N && p0 > 0) ? sp[nn] : 0.f;
   }
   const float dtb = dt_bias[c], dd = Dv[c];
-  for (int t = 0; t < n; ++t) {
-    const long tok = q0 + t;
+  for (int t0 = 0; t0 < n; t0 += 16) {
+    const int nt = min(16, n - t0);
+    __syncthreads();                    // the previous group's rows are consumed
+    for (int e = tid; e < nt * N2; e += 256) {
+      const int tt = e / N2, k = e - tt * N2;
+      bcs[e] = ldf(dbc + (long)(q0 + t0 + tt) * ldd + dt_rank + k);
+    }
+    const long tok = q0 + t0 + min(sub, nt - 1);
     const float raw = ldf(dt_raw + tok * C + c) + dtb;
-    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
-    const float xv = ldf(xc + tok * C + c);
-    const T* bc = dbc + tok * ldd + dt_rank;
-    float acc = 0.f;
+    const float dt_m = raw > 20.f ? raw : log1pf(expf(raw));
+    const float x_m = ldf(xc + tok * C + c);
+    const float z_m = ldf(xz + tok * ldz + C + c);
+    __syncthreads();
+    float y_m = 0.f;
+    for (int u = 0; u < nt; ++u) {
+      const float dt = __shfl(dt_m, u, 16), xv = __shfl(x_m, u, 16);
+      const float* bc = bcs + u * N2;
+      float acc = 0.f;
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-      const int nn = sub + 16 * i;
-      if (nn < N) {
-        S[i] = expf(dt * a[i]) * S[i] + dt * xv * ldf(bc + nn);
-        acc += S[i] * ldf(bc + N + nn);
+      for (int i = 0; i < NS; ++i) {
+        const int nn = sub + 16 * i;
+        if (nn < N) {
+          S[i] = fastexp<T>::f(dt * a[i]) * S[i] + dt * xv * bc[nn];
+          acc += S[i] * bc[N + nn];
+        }
       }
-    }
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 16);
-    if (sub == 0) {
-      const float z = ldf(xz + tok * ldz + C + c);
-      stf(out + tok * C + c, (acc + dd * xv) * silu_f(z));
+      for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 16);
+      if (sub == u) y_m = acc;
     }
+    if (live && sub < nt) stf(out + tok * C + c, (y_m + dd * x_m) * silu_f(z_m));
   }
+  if (!live) return;
 #pragma unroll
   for (int i = 0; i < NS; ++i) {
     const int nn = sub + 16 * i;
@@ -251,6 +277,174 @@ __global__ void __launch_bounds__(256) retention_kernel(const T* __restrict__ qk
   }
   __syncthreads();
   for (int e = tid; e < d * dv; e += 256) sg[e] = S[e];
+}
+
+// ---------------------------------------------------------------- retention, chunked (prompt portions)
+// One workgroup per (head, 32-column slice of the value dim, sequence); tokens in chunks of 32.
+// With the chunk's rotated q / k (k scaled) and v slice in LDS and g = decay:
+//   A[t][s] = g^(t-s) q_t . k_s  (s <= t)            scores inside the chunk, f32
+//   o_t     = g^(t+1) q_t^T S + sum_s A[t][s] v_s     S: the state slice before the chunk
+//   S      <- g^n S + sum_s g^(n-1-s) k_s v_s^T       n tokens in the chunk
+// The raw outputs go to an f32 buffer; retention_finish norms each head and applies the gate.
+constexpr int RC_T = 32, RC_V = 32;
+
+template <typename T>
+__global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restrict__ qkvg, long ld, int H, int d, int dv,
+                                                              const float* __restrict__ cos_sin, int tab_w, int rot,
+                                                              const float* __restrict__ decay, float* __restrict__ state,
+                                                              const int* __restrict__ qstart, const int* __restrict__ qlen,
+                                                              const int* __restrict__ ctx, const int* __restrict__ rows,
+                                                              float* __restrict__ raw) {
+  extern __shared__ float sm[];
+  const int h = blockIdx.x, v0 = blockIdx.y * RC_V, s = blockIdx.z;
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  const int nv = min(RC_V, dv - v0), dp = d + 1;
+  float* Qs = sm;                       // [RC_T][d + 1]
+  float* Ks = Qs + RC_T * dp;           // [RC_T][d + 1]
+  float* Vs = Ks + RC_T * dp;           // [RC_T][RC_V]
+  float* As = Vs + RC_T * RC_V;         // [RC_T][RC_T + 1]
+  float* S = As + RC_T * (RC_T + 1);    // [d][RC_V]
+  float* gp = S + d * RC_V;             // [RC_T + 1] powers of the decay
+  const int tid = threadIdx.x;
+  float* sg = state + ((long)rows[s] * H + h) * d * dv;
+  for (int e = tid; e < d * RC_V; e += 256) {
+    const int i = e / RC_V, j = e % RC_V;
+    S[e] = (p0 > 0 && j < nv) ? sg[(long)i * dv + v0 + j] : 0.f;
+  }
+  const float dec = decay[h], kscale = 1.f / sqrtf((float)d);
+  if (tid <= RC_T) gp[tid] = powf(dec, (float)tid);
+  const int half = rot >> 1;
+  const long oq = (long)h * d, ok = (long)H * d + (long)h * d, ov = 2L * H * d + (long)h * dv + v0;
+  for (int t0 = 0; t0 < n; t0 += RC_T) {
+    const int nt = min(RC_T, n - t0);
+    __syncthreads();   // state loaded / previous chunk's state update done
+    for (int e = tid; e < RC_T * d; e += 256) {
+      const int tt = e / d, i = e % d;
+      float qv = 0.f, kv = 0.f;
+      if (tt < nt) {
+        const T* r = qkvg + (long)(q0 + t0 + tt) * ld;
+        qv = ldf(r + oq + i);
+        kv = ldf(r + ok + i);
+        if (i < rot) {
+          const int f = i < half ? i : i - half;
+          const float* cs = cos_sin + (long)(p0 + t0 + tt) * tab_w;
+          const float c = cs[f], sn = cs[half + f];
+          const int pi = i < half ? i + half : i - half;
+          const float qp = ldf(r + oq + pi), kp = ldf(r + ok + pi);
+          qv = i < half ? qv * c - qp * sn : qv * c + qp * sn;
+          kv = i < half ? kv * c - kp * sn : kv * c + kp * sn;
+        }
+      }
+      Qs[tt * dp + i] = qv;
+      Ks[tt * dp + i] = kv * kscale;
+    }
+    for (int e = tid; e < RC_T * RC_V; e += 256) {
+      const int tt = e / RC_V, j = e % RC_V;
+      Vs[e] = (tt < nt && j < nv) ? ldf(qkvg + (long)(q0 + t0 + tt) * ld + ov + j) : 0.f;
+    }
+    __syncthreads();
+    // scores inside the chunk: thread (t, 4 keys u0..u0+3); one q read serves four sums
+    {
+      const int t = tid >> 3, u0 = (tid & 7) * 4;
+      float a4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (u0 <= t) {
+        const float* q = Qs + t * dp;
+        const float* k = Ks + u0 * dp;
+#pragma unroll 4
+        for (int i = 0; i < d; ++i) {
+          const float qv = q[i];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) a4[x] += qv * k[x * dp + i];
+        }
+      }
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int u = u0 + x;
+        As[t * (RC_T + 1) + u] = (u <= t && t < nt) ? a4[x] * gp[t - u] : 0.f;
+      }
+    }
+    __syncthreads();
+    // outputs: thread (t, 4 value columns j0..j0+3)
+    {
+      const int t = tid >> 3, j0 = (tid & 7) * 4;
+      const float* q = Qs + t * dp;
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+      for (int i = 0; i < d; ++i) {
+        const float qv = q[i];
+        const float4 sv = *reinterpret_cast<const float4*>(S + i * RC_V + j0);
+        o4[0] += qv * sv.x; o4[1] += qv * sv.y; o4[2] += qv * sv.z; o4[3] += qv * sv.w;
+      }
+      const float g1 = gp[t + 1];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) o4[x] *= g1;
+      const float* a = As + t * (RC_T + 1);
+      for (int u = 0; u <= t; ++u) {
+        const float av = a[u];
+        const float4 vv = *reinterpret_cast<const float4*>(Vs + u * RC_V + j0);
+        o4[0] += av * vv.x; o4[1] += av * vv.y; o4[2] += av * vv.z; o4[3] += av * vv.w;
+      }
+      if (t < nt) {
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+          if (j0 + x < nv) raw[((long)(q0 + t0 + t) * H + h) * dv + v0 + j0 + x] = o4[x];
+      }
+    }
+    __syncthreads();
+    // state: thread (row i, 16 value columns); rows in passes of 128
+    {
+      const int jb = (tid & 1) * 16;
+      const float gn = gp[nt];
+      for (int i = tid >> 1; i < d; i += 128) {
+        float acc[16];
+#pragma unroll
+        for (int x = 0; x < 16; ++x) acc[x] = gn * S[i * RC_V + jb + x];
+        for (int u = 0; u < nt; ++u) {
+          const float kv = gp[nt - 1 - u] * Ks[u * dp + i];
+          const float* v = Vs + u * RC_V + jb;
+#pragma unroll
+          for (int x = 0; x < 16; x += 4) {
+            const float4 vv = *reinterpret_cast<const float4*>(v + x);
+            acc[x] += kv * vv.x; acc[x + 1] += kv * vv.y; acc[x + 2] += kv * vv.z; acc[x + 3] += kv * vv.w;
+          }
+        }
+#pragma unroll
+        for (int x = 0; x < 16; ++x) S[i * RC_V + jb + x] = acc[x];
+      }
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < d * RC_V; e += 256) {
+    const int i = e / RC_V, j = e % RC_V;
+    if (j < nv) sg[(long)i * dv + v0 + j] = S[e];
+  }
+}
+
+// unit-RMS heads and the SiLU gate over the raw outputs: one wave per (token, head)
+template <typename T>
+__global__ void __launch_bounds__(256) retention_finish_kernel(const float* __restrict__ raw, const T* __restrict__ qkvg,
+                                                               long ld, int H, int d, int dv, float eps,
+                                                               const int* __restrict__ qstart, const int* __restrict__ qlen,
+                                                               int S, T* __restrict__ out, long rows_total) {
+  const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows_total) return;
+  const int lane = threadIdx.x & 63;
+  const long tok = r / H;
+  const int h = (int)(r % H);
+  // tokens of no sequence (graph padding) keep their zeros
+  bool live = false;
+  for (int s = 0; s < S; ++s) live |= tok >= qstart[s] && tok < qstart[s] + qlen[s];
+  if (!live) return;
+  const float* o = raw + r * dv;
+  float ss = 0.f;
+  for (int j = lane; j < dv; j += 64) ss += o[j] * o[j];
+  ss = wave_sum(ss);
+  const float rs = 1.f / sqrtf(ss / (float)dv + eps);
+  const long og = 2L * H * d + (long)H * dv + (long)h * dv;
+  for (int j = lane; j < dv; j += 64)
+    stf(out + tok * ((long)H * dv) + (long)h * dv + j, o[j] * rs * silu_f(ldf(qkvg + tok * ld + og + j)));
 }
 
 // ---------------------------------------------------------------- squared ReLU, dense gate
@@ -369,6 +563,38 @@ extern "C" int dllm_retention(const void* qkvg, long ld, int f32, int H, int d, 
     if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(retention_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
                        decay, state, eps, qstart, qlen, ctx, rows, (u16*)out, lj);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" long dllm_retention_chunk_lds(int d) {
+  return 4L * (2L * RC_T * (d + 1) + RC_T * RC_V + RC_T * (RC_T + 1) + (long)d * RC_V + RC_T + 1);
+}
+
+// Chunked form for prompt portions: `raw` is an f32 scratch [T, H, dv].
+extern "C" int dllm_retention_chunked(const void* qkvg, long ld, int f32, int H, int d, int dv, const float* cos_sin,
+                                      int tab_w, int rot, const float* decay, float* state, float eps, const int* qstart,
+                                      const int* qlen, const int* ctx, const int* rows, float* raw, void* out, int S,
+                                      long T, hipStream_t st) {
+  if (S <= 0 || T <= 0) return 0;
+  if (rot < 0 || rot > d || (rot & 1) || rot > tab_w) return -1;
+  const long lds = dllm_retention_chunk_lds(d);
+  if (lds > 150 * 1024) return -2;
+  const dim3 g(H, (dv + RC_V - 1) / RC_V, S);
+  const long rows_total = T * H;
+  const dim3 gf((unsigned)((rows_total + 3) / 4));
+  if (f32) {
+    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_chunk_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(retention_chunk_kernel<float>, g, dim3(256), lds, st, (const float*)qkvg, ld, H, d, dv, cos_sin, tab_w,
+                       rot, decay, state, qstart, qlen, ctx, rows, raw);
+    hipLaunchKernelGGL(retention_finish_kernel<float>, gf, dim3(256), 0, st, raw, (const float*)qkvg, ld, H, d, dv, eps, qstart,
+                       qlen, S, (float*)out, rows_total);
+  } else {
+    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_chunk_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(retention_chunk_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
+                       decay, state, qstart, qlen, ctx, rows, raw);
+    hipLaunchKernelGGL(retention_finish_kernel<u16>, gf, dim3(256), 0, st, raw, (const u16*)qkvg, ld, H, d, dv, eps, qstart, qlen,
+                       S, (u16*)out, rows_total);
   }
   return (int)hipGetLastError();
 }

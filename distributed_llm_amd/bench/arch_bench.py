@@ -1,0 +1,210 @@
+"""Layer-list (Filevik) models beside the closest Llama-family model at equal size: prefill and
+decode throughput through the engine, and the time of each mixer kernel against its roofline.
+
+``python bench.py --arch-bench [--arch-size s|m]`` (random weights, synthetic tokens).  The default
+bench workload and its JSON contract are untouched; this prints one JSON object of its own.
+
+Sizes: width / layers of a small and a mid-size decoder.  The Filevik stack cycles mamba1 ->
+retention -> latent attention, each with routed squared-ReLU experts and a shared expert; the
+comparison model is a Mixtral-style Llama (grouped-query attention + SwiGLU experts) with the same
+width, layer count, expert count / top-k and per-token expert width.
+"""
+from __future__ import annotations
+
+import json
+import time
+from typing import Dict, List
+
+import torch
+
+PEAK_BW = 8.0e12          # HBM3E bytes/s
+PEAK_BF16 = 2.5e15        # dense bf16 MFMA flop/s
+PEAK_F32 = 157e12         # f32 vector flop/s
+
+SIZES = {
+    "s": dict(width=1024, layers=6, inner=2048, state=16, dt_rank=64, conv=4, heads=8, dim=64, vdim=128, rot=64,
+              lat_heads=16, lat_dim=64, lat_rot=32, lat_v=64, kv_rank=256, q_rank=768, experts=8, top=2, ff=1024,
+              shared=1024, vocab=32000),
+    "m": dict(width=2048, layers=12, inner=4096, state=16, dt_rank=128, conv=4, heads=16, dim=128, vdim=128, rot=64,
+              lat_heads=16, lat_dim=128, lat_rot=64, lat_v=128, kv_rank=512, q_rank=1536, experts=8, top=2, ff=2048,
+              shared=2048, vocab=32000),
+}
+
+
+def filevik_raw(z: dict) -> dict:
+    mlp = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"], "scale": 1.0}, "expert": {"ff": z["ff"]},
+           "shared": {"ff": z["shared"]}}
+    kinds = [
+        {"type": "mamba1", "mixer": {"inner": z["inner"], "state": z["state"], "dt_rank": z["dt_rank"], "conv": z["conv"]}},
+        {"type": "retention", "mixer": {"heads": z["heads"], "dim": z["dim"], "vdim": z["vdim"],
+                                        "decay": [1.0 - 2.0 ** (-5 - i % 4) for i in range(z["heads"])],
+                                        "rot": {"dims": z["rot"], "base": 10000.0}}},
+        {"type": "latent_attention", "mixer": {"heads": z["lat_heads"], "dim": z["lat_dim"], "rot_dim": z["lat_rot"],
+                                               "vdim": z["lat_v"], "kv_rank": z["kv_rank"], "q_rank": z["q_rank"],
+                                               "scale": (z["lat_dim"] + z["lat_rot"]) ** -0.5,
+                                               "rot": {"dims": z["lat_rot"], "base": 10000.0}}},
+    ]
+    return {"architecture": "Filevik", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "layers": [dict(kinds[i % 3], mlp=mlp) for i in range(z["layers"])]}
+
+
+def llama_twin(z: dict):
+    from ..models.configs import ModelConfig
+    return ModelConfig(f"moe-llama-{z['width']}", z["width"], z["layers"], z["width"] // 64, max(1, z["width"] // 256), 64,
+                       z["ff"] * 3 // 2 // 64 * 64, z["vocab"], 10000.0, 1e-6, 16384, n_experts=z["experts"],
+                       experts_per_token=z["top"])
+
+
+def _timed(fn, iters: int = 5) -> float:
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters * 1e-3
+
+
+def engine_throughput(model, prompts: List[int], batches: List[int], ctx: int, new: int, rows: int) -> Dict[str, float]:
+    from ..engine.llm_engine import LLMEngine
+    from ..engine.sampling import SamplingParams
+    eng = LLMEngine(model, device="cuda", kv_cache_gb=8.0, max_num_seqs=rows, max_model_len=max(max(prompts), ctx) + new + 64,
+                    prefix_cache=False)
+    out: Dict[str, float] = {}
+    g = torch.Generator().manual_seed(0)
+    V = eng.cfg.vocab
+    mk = lambda n, L: [torch.randint(3, V, (L,), generator=g).tolist() for _ in range(n)]
+    one = SamplingParams(max_new_tokens=1, temperature=0.0, ignore_eos=True)
+    for L in prompts:                      # prefill: whole prompts, one generated token each
+        n = max(1, min(rows, 16384 // L))
+        eng.generate(mk(n, L), one)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.generate(mk(n, L), one)
+        torch.cuda.synchronize()
+        out[f"prefill_tok_s_L{L}"] = round(n * L / (time.perf_counter() - t0), 1)
+    for B in batches:                      # decode: B sequences of ctx tokens, `new` tokens each
+        sp = SamplingParams(max_new_tokens=new, temperature=0.0, ignore_eos=True)
+        eng.generate(mk(B, ctx), SamplingParams(max_new_tokens=4, temperature=0.0, ignore_eos=True))
+        st0 = dict(eng.timers)
+        s0 = dict(eng.steps)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.generate(mk(B, ctx), sp)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0 - (eng.timers["prefill"] - st0["prefill"])
+        steps = eng.steps["decode"] - s0["decode"]
+        out[f"decode_tok_s_B{B}"] = round(B * new / dt, 1)
+        out[f"decode_ms_step_B{B}"] = round(dt / max(1, steps) * 1e3, 3)
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
+def kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 2048) -> Dict[str, dict]:
+    """Each mixer kernel alone (bf16): prefill of one T-token sequence, decode of B sequences at
+    ``ctx``; time, the bound resource's minimum time, and their ratio."""
+    from .. import ops
+    from ..ops import seqmix
+    dev, bf = "cuda", torch.bfloat16
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, bytes_, flops, peak_flops):
+        floor = max(bytes_ / PEAK_BW, flops / peak_flops)
+        res[name] = {"us": round(sec * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "x_roofline": round(sec / floor, 1),
+                     "bound": "memory" if bytes_ / PEAK_BW >= flops / peak_flops else "compute"}
+
+    for tag, qlens, starts in (("prefill", [T], [0]), ("decode", [1] * B, [ctx] * B)):
+        n = sum(qlens)
+        S = len(qlens)
+        qstart = i32([sum(qlens[:i]) for i in range(S)])
+        qlen, cx, rows = i32(qlens), i32([a + b for a, b in zip(starts, qlens)]), i32(list(range(S)))
+        pos = i32([p for a, m in zip(starts, qlens) for p in range(a, a + m)])
+        # selective scan (+ conv)
+        C, N, R, K = z["inner"], z["state"], z["dt_rank"], z["conv"]
+        xz = torch.randn(n, 2 * C, device=dev).to(bf)
+        conv_s, ssm = torch.zeros(S, K - 1, C, device=dev, dtype=bf), torch.zeros(S, C, N, device=dev)
+        w, b_ = torch.randn(C, K, device=dev), torch.zeros(C, device=dev)
+        xc = seqmix.causal_conv_silu(xz, w, b_, conv_s, qstart, qlen, cx, rows)
+        dbc = torch.randn(n, R + 2 * N, device=dev).to(bf)
+        dtr, dtb = torch.randn(n, C, device=dev).to(bf), torch.zeros(C, device=dev)
+        A, D = -torch.rand(C, N, device=dev), torch.ones(C, device=dev)
+        rec(f"conv_{tag}", _timed(lambda: seqmix.causal_conv_silu(xz, w, b_, conv_s, qstart, qlen, cx, rows)),
+            n * C * 4 + (S * (K - 1) * C * 2 if tag == "decode" else 0), n * C * 2 * K, PEAK_F32)
+        rec(f"scan_{tag}", _timed(lambda: seqmix.selective_scan(xc, dtr, dtb, A, dbc, R, D, xz, ssm, conv_s, qstart, qlen, cx, rows)),
+            n * C * 8 + (S * C * N * 8 if tag == "decode" else 0), n * C * N * 12, PEAK_F32)
+        # retention
+        H, d, dv = z["heads"], z["dim"], z["vdim"]
+        qkvg = torch.randn(n, 2 * H * d + 2 * H * dv, device=dev).to(bf)
+        table = ops.rope_cos_sin(ctx + T + 8, z["rot"], 10000.0, dev)
+        dec, st = torch.full((H,), 0.98, device=dev), torch.zeros(S, H, d, dv, device=dev)
+        rec(f"retention_{tag}", _timed(lambda: seqmix.retention(qkvg, H, d, dv, table, z["rot"], dec, st, 1e-6, pos, qstart, qlen, cx, rows)),
+            n * (2 * H * d + 3 * H * dv) * 2 + (S * H * d * dv * 8 if tag == "decode" else 0),
+            n * H * d * dv * 4 if tag == "decode" else n * H * (4 * d * dv + 2 * 64 * (d + dv)), PEAK_F32)
+        # latent attention
+        Hl, r, dr, dl = z["lat_heads"], z["kv_rank"], z["lat_rot"], z["lat_dim"]
+        nb = (max(cx.tolist()) + 15) // 16
+        bt = torch.arange(S * nb, dtype=torch.int32, device=dev).view(S, nb)
+        cache = (torch.randn(S * nb, 16, r + dr, device=dev) * 0.3).to(bf)
+        qa, q = (torch.randn(Hl, n, r, device=dev) * 0.3).to(bf), torch.randn(n, Hl * (dl + dr), device=dev).to(bf)
+        tab2 = ops.rope_cos_sin(ctx + T + 8, dr, 10000.0, dev)
+        from ..models.llama import AttnMeta
+        meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=cx, tile_seq=None, tile_tok0=None,
+                        last_idx=None, host_qlen=qlens)
+        ts, tt = meta.latent_tiles(Hl, dev)
+        keys = sum((a + (m + 1) / 2) * m for a, m in zip(starts, qlens))     # causal (query, key) pairs
+        rec(f"latent_attention_{tag}",
+            _timed(lambda: seqmix.latent_attention(qa, q, dl, dr, pos, tab2, cache, bt, qstart, qlen, cx, ts, tt, 0.1), 3),
+            (sum(a + m for a, m in zip(starts, qlens)) * (r + dr) * 2 + n * Hl * r * 4),
+            keys * Hl * (2 * (r + dr) + 2 * r), PEAK_BF16)
+    return res
+
+
+def llama_kernel_rooflines(T: int = 4096, B: int = 64, ctx: int = 2048, nq: int = 32, nkv: int = 8, d: int = 64) -> Dict[str, dict]:
+    """The comparison model's attention kernels at the same token counts."""
+    from .. import ops
+    dev, bf = "cuda", torch.bfloat16
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    res = {}
+    for tag, qlens, starts in (("prefill", [T], [0]), ("decode", [1] * B, [ctx] * B)):
+        n, S = sum(qlens), len(qlens)
+        cx = [a + m for a, m in zip(starts, qlens)]
+        nb = (max(cx) + 15) // 16
+        bt = torch.arange(S * nb, dtype=torch.int32, device=dev).view(S, nb)
+        kc = (torch.randn(S * nb, nkv, 16, d, device=dev) * 0.3).to(bf)
+        vc = (torch.randn(S * nb, nkv, d, 16, device=dev) * 0.3).to(bf)
+        q = torch.randn(n, nq, d, device=dev).to(bf)
+        qstart = i32([sum(qlens[:i]) for i in range(S)])
+        G = nq // nkv
+        if tag == "prefill" and ops.flash_supported(d, G, nb):
+            ts, tt = ops.flash_tiles(qlens, G)
+            fn = lambda: ops.flash_attention(q, kc, vc, bt, qstart, i32(qlens), i32(cx), i32(ts), i32(tt), max_ctx=max(cx))
+        else:
+            ts, tt = ops.build_tiles(qlens, G)
+            fn = lambda: ops.paged_attention(q, kc, vc, bt, qstart, i32(qlens), i32(cx), i32(ts), i32(tt))
+        sec = _timed(fn)
+        keys = sum((a + (m + 1) / 2) * m for a, m in zip(starts, qlens))
+        bytes_, flops = sum(cx) * nkv * d * 4 + n * nq * d * 4, keys * nq * d * 4
+        floor = max(bytes_ / PEAK_BW, flops / PEAK_BF16)
+        res[f"attention_{tag}"] = {"us": round(sec * 1e6, 1), "roofline_us": round(floor * 1e6, 2),
+                                   "x_roofline": round(sec / floor, 1),
+                                   "bound": "memory" if bytes_ / PEAK_BW >= flops / PEAK_BF16 else "compute"}
+    return res
+
+
+def run(size: str = "s", kernels_only: bool = False) -> dict:
+    from ..models.configs import filevik_config
+    z = SIZES[size]
+    out = {"bench": "arch", "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}
+    out["filevik_kernels"] = kernel_rooflines(z)
+    out["llama_kernels"] = llama_kernel_rooflines()
+    if not kernels_only:
+        fcfg = filevik_config(filevik_raw(z), name=f"filevik-{size}")
+        prompts, batches = [512, 2048], [1, 16, 64]
+        out["filevik"] = engine_throughput(fcfg, prompts, batches, ctx=1024, new=32, rows=64)
+        out["moe_llama"] = engine_throughput(llama_twin(z), prompts, batches, ctx=1024, new=32, rows=64)
+    print(json.dumps(out))
+    return out

@@ -65,15 +65,23 @@ def selective_scan(xc, dt_raw, dt_bias, A, dbc, dt_rank, D, xz, ssm_state, conv_
     return out
 
 
+RETENTION_CHUNK_MIN = 4    # average new tokens per sequence from which the chunked kernel runs
+
+
 def retention(qkvg, heads, dim, vdim, cos_sin, rot_dims, decay, state, eps, positions, qstart, qlen, ctx,
-              rows) -> torch.Tensor:
+              rows, chunked: Optional[bool] = None) -> torch.Tensor:
+    """``chunked`` (GPU): the chunk-parallel kernel (prompt portions) or the token-by-token one
+    (decode steps); default by the step's tokens per sequence.  Same results either way."""
     ext = _native(qkvg)
     if ext is None:
         return ref.retention(qkvg, heads, dim, vdim, cos_sin, rot_dims, decay, state, eps, positions, qstart, qlen,
                              ctx, rows)
     out = torch.zeros((qkvg.shape[0], heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    if chunked is None:
+        chunked = qkvg.shape[0] >= RETENTION_CHUNK_MIN * qstart.numel()
+    raw = torch.empty((qkvg.shape[0], heads, vdim), dtype=torch.float32, device=qkvg.device) if chunked else None
     ext.retention(qkvg, int(heads), int(dim), int(vdim), cos_sin, int(rot_dims), decay, state, float(eps), positions,
-                  qstart, qlen, ctx, rows, out)
+                  qstart, qlen, ctx, rows, out, raw)
     return out
 
 

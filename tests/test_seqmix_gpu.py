@@ -93,8 +93,9 @@ def test_conv_and_scan(dt, case, C, N, K, R):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("chunked", [False, True])
 @pytest.mark.parametrize("H,d,dv,rot", [(2, 64, 32, 64), (3, 32, 24, 16), (1, 16, 80, 0), (4, 128, 128, 64)])
-def test_retention(dt, case, H, d, dv, rot):
+def test_retention(dt, case, H, d, dv, rot, chunked):
     torch.manual_seed(2)
     qlens, starts = case
     T, qstart, qlen, ctx, rows, pos = batch(qlens, starts)
@@ -103,7 +104,7 @@ def test_retention(dt, case, H, d, dv, rot):
     decay = torch.tensor([1.0 - 2.0 ** (-2 - h) for h in range(H)], device=DEV)
     st0 = torch.randn(len(qlens) + 1, H, d, dv, device=DEV)
     s1, s2 = st0.clone(), st0.clone()
-    o1 = seqmix.retention(qkvg, H, d, dv, table, rot, decay, s1, 1e-6, pos, qstart, qlen, ctx, rows)
+    o1 = seqmix.retention(qkvg, H, d, dv, table, rot, decay, s1, 1e-6, pos, qstart, qlen, ctx, rows, chunked=chunked)
     o2 = ref.retention(qkvg, H, d, dv, table, rot, decay, s2, 1e-6, pos, qstart, qlen, ctx, rows)
     torch.testing.assert_close(o1.float(), o2.float(), **tol(dt))
     torch.testing.assert_close(s1, s2, atol=2e-4, rtol=2e-4)
