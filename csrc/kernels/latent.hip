@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     const float* __restrict__ cos_sin, int tab_w, const T* __restrict__ cache, const int* __restrict__ bt, int bt_w,
     const int* __restrict__ qstart, const int* __restrict__ qlen, const int* __restrict__ ctx,
     const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, T* __restrict__ out, int KT,
-    int tpe) {
+    int tpe, int kstride, int vec) {
   extern __shared__ float sm[];
   const int entry = blockIdx.y;
   const int s = tile_seq[entry];
@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
   const int row0 = blockIdx.x * LROWS;
   if (row0 >= nrows) return;
   const int q0 = qstart[s], p0 = ctx[s] - n;
-  const int Dp = rank + rot, kstride = Dp | 1;
+  const int Dp = rank + rot;
   float* qsh = sm;                              // [16][Dp]
   float* ksh = qsh + LROWS * Dp;                // [KT][kstride]
   float* psh = ksh + KT * kstride;              // [16][64]
@@ -124,10 +124,11 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
   for (int k0 = 0; k0 < kmax; k0 += KT) {
     const int nk = min(KT, kmax - k0);
     __syncthreads();   // the previous tile is consumed (and the queries are staged)
-    for (int e = tid; e < nk * Dp; e += 256) {
-      const int kk = e / Dp, c = e % Dp, kidx = k0 + kk;
-      const long slot = (long)btr[kidx >> 4] * 16 + (kidx & 15);
-      ksh[kk * kstride + c] = ldf(cache + slot * Dp + c);
+    for (int kk = wave; kk < nk; kk += 4) {          // a wave per key row, lanes along the row
+      const int kidx = k0 + kk;
+      const T* src = cache + ((long)btr[kidx >> 4] * 16 + (kidx & 15)) * Dp;
+      float* dst = ksh + kk * kstride;
+      for (int c = lane; c < Dp; c += 64) dst[c] = ldf(src + c);
     }
     __syncthreads();
     // phase 1: lane = key
@@ -135,10 +136,22 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     if (lane < nk) {
       const float* kr = ksh + lane * kstride;
       const float* qr = qsh + (wave * 4) * Dp;
-      for (int c = 0; c < Dp; ++c) {
-        const float kv = kr[c];
+      if (vec) {          // 16-byte LDS reads: rows are 16-byte aligned, kstride / 4 is odd (no bank conflicts)
+#pragma unroll 2
+        for (int c = 0; c < Dp; c += 4) {
+          const float4 kv = *reinterpret_cast<const float4*>(kr + c);
 #pragma unroll
-        for (int a = 0; a < 4; ++a) sc[a] += qr[a * Dp + c] * kv;
+          for (int a = 0; a < 4; ++a) {
+            const float4 qv = *reinterpret_cast<const float4*>(qr + a * Dp + c);
+            sc[a] += qv.x * kv.x + qv.y * kv.y + qv.z * kv.z + qv.w * kv.w;
+          }
+        }
+      } else {
+        for (int c = 0; c < Dp; ++c) {
+          const float kv = kr[c];
+#pragma unroll
+          for (int a = 0; a < 4; ++a) sc[a] += qr[a * Dp + c] * kv;
+        }
       }
     }
     float alpha[4];
@@ -214,14 +227,15 @@ template <typename T>
 int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T* q, long ldq, int H, int dim, int rot,
                   int rank, long Ttot, const float* cos_sin, int tab_w, const T* cache, const int* bt, int bt_w,
                   const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
-                  float scale, T* out, int KT, int tpe) {
+                  float scale, T* out, int KT, int tpe, int kstride, int vec) {
 #define LAT(RI)                                                                                                        \
   do {                                                                                                                 \
     if (lds > 48 * 1024)                                                                                               \
       hipFuncSetAttribute((const void*)latent_attention_kernel<T, RI>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
                           (int)lds);                                                                                   \
     hipLaunchKernelGGL((latent_attention_kernel<T, RI>), g, dim3(256), lds, st, qa, q, ldq, H, dim, rot, rank, Ttot,   \
-                       cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT, tpe);  \
+                       cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT, tpe,   \
+                       kstride, vec);                                                                                  \
   } while (0)
   if (ri <= 1) LAT(1); else if (ri <= 2) LAT(2); else if (ri <= 4) LAT(4); else LAT(8);
 #undef LAT
@@ -235,7 +249,10 @@ extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, in
                                      const int* tile_tok0, int n_entries, float scale, void* out, hipStream_t st) {
   if (n_entries <= 0 || Ttot <= 0) return 0;
   if (rank < 1 || rank > 512 || rot < 0 || (rot & 1) || rot > tab_w || H < 1) return -1;
-  const int Dp = rank + rot, kstride = Dp | 1;
+  // key rows in LDS: an odd stride for 4-byte reads; when the row length is a multiple of 4 a stride
+  // that is 4 x odd, so a lane's 16-byte reads are aligned and spread over all banks
+  const int Dp = rank + rot, vec = (Dp & 3) == 0;
+  const int kstride = vec ? (((Dp >> 2) & 1) ? Dp : Dp + 4) : (Dp | 1);
   int KT = 64;
   while (KT > 8 && 4L * (LROWS * Dp + (long)KT * kstride + LROWS * 64) > 140 * 1024) KT >>= 1;
   const long lds = 4L * (LROWS * Dp + (long)KT * kstride + LROWS * 64);
@@ -246,7 +263,7 @@ extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, in
   if (f32)
     return launch_latent<float>(ri, g, lds, st, (const float*)qa, (const float*)q, ldq, H, dim, rot, rank, Ttot, cos_sin,
                                 tab_w, (const float*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale,
-                                (float*)out, KT, tpe);
+                                (float*)out, KT, tpe, kstride, vec);
   return launch_latent<u16>(ri, g, lds, st, (const u16*)qa, (const u16*)q, ldq, H, dim, rot, rank, Ttot, cos_sin, tab_w,
-                            (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KT, tpe);
+                            (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KT, tpe, kstride, vec);
 }

@@ -100,6 +100,15 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x,
 // same rows), and lane `sub` of a channel prepares token `sub` of the group (softplus step, input,
 // gate) and finishes it (skip term, SiLU gate, store), so the serial part of a token is only the
 // state update itself: NS exponentials and multiply-adds, a 16-lane sum, two broadcasts.
+// sum over the 16 lanes of a DPP row (rotations inside the row): every lane ends with the total
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));  // row_ror:8
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));  // row_ror:4
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));  // row_ror:2
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));  // row_ror:1
+  return v;
+}
+
 template <typename T> struct fastexp;
 template <> struct fastexp<u16> { static __device__ __forceinline__ float f(float x) { return __expf(x); } };
 template <> struct fastexp<float> { static __device__ __forceinline__ float f(float x) { return expf(x); } };
@@ -114,6 +123,7 @@ __global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, con
                                                    const int* __restrict__ ctx, const int* __restrict__ rows,
                                                    T* __restrict__ out, int C, int N) {
   __shared__ float bcs[16 * 256];       // [16 tokens][2N], N <= 128
+  __shared__ float dts[256], xs[256];   // [16 channels][16 tokens]: step size and input of the group's tokens
   const int s = blockIdx.y;
   const int n = qlen[s];
   if (n <= 0) return;                   // the whole workgroup
@@ -144,10 +154,14 @@ __global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, con
     const float dt_m = raw > 20.f ? raw : log1pf(expf(raw));
     const float x_m = ldf(xc + tok * C + c);
     const float z_m = ldf(xz + tok * ldz + C + c);
+    dts[tid] = dt_m;
+    xs[tid] = x_m;
     __syncthreads();
     float y_m = 0.f;
+    const int g0 = tid & ~15;
+#pragma unroll 4
     for (int u = 0; u < nt; ++u) {
-      const float dt = __shfl(dt_m, u, 16), xv = __shfl(x_m, u, 16);
+      const float dt = dts[g0 + u], xv = xs[g0 + u];   // independent of the state: read ahead
       const float* bc = bcs + u * N2;
       float acc = 0.f;
 #pragma unroll
@@ -158,8 +172,7 @@ __global__ void __launch_bounds__(256) scan_kernel(const T* __restrict__ xc, con
           acc += S[i] * bc[N + nn];
         }
       }
-#pragma unroll
-      for (int o = 8; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 16);
+      acc = row16_sum(acc);
       if (sub == u) y_m = acc;
     }
     if (live && sub < nt) stf(out + tok * C + c, (y_m + dd * x_m) * silu_f(z_m));
