@@ -67,7 +67,7 @@ int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, 
                          void*, int, hipStream_t);
 int dllm_latent_attention(const void*, const void*, long, int, int, int, int, int, long, const float*, int, const void*,
                           const int*, int, const int*, const int*, const int*, const int*, const int*, int, float, void*,
-                          hipStream_t);
+                          int, float*, float*, hipStream_t);
 int dllm_car_alloc(long, void**);
 int dllm_car_get_handle(void*, char*);
 int dllm_car_handle_size();
@@ -1483,7 +1483,8 @@ void latent_kv_write(torch::Tensor ckv, int64_t rank, torch::Tensor w, double ep
 
 void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t rot, torch::Tensor pos, torch::Tensor cos_sin,
                       torch::Tensor cache, torch::Tensor bt, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
-                      torch::Tensor tile_seq, torch::Tensor tile_tok0, double scale, torch::Tensor out) {
+                      torch::Tensor tile_seq, torch::Tensor tile_tok0, double scale, torch::Tensor out, int64_t splits,
+                      c10::optional<torch::Tensor> part_o, c10::optional<torch::Tensor> part_ml) {
   const bool f = act_f32(qa, "qa");
   TORCH_CHECK(qa.dim() == 3 && qa.is_contiguous(), "qa [H, T, rank] contiguous");
   const int64_t H = qa.size(0), T = qa.size(1), rank = qa.size(2);
@@ -1503,11 +1504,22 @@ void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t ro
   TORCH_CHECK(rank <= 512, "latent rank <= 512");
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == qa.scalar_type() && out.is_contiguous() && out.sizes() == qa.sizes(),
               "out like qa");
+  float *po = nullptr, *pml = nullptr;
+  TORCH_CHECK(splits >= 1 && splits <= 64, "splits in [1, 64]");
+  if (splits > 1) {
+    TORCH_CHECK(part_o && part_ml, "split partial buffers");
+    check_f32(*part_o, "part_o");
+    check_f32(*part_ml, "part_ml");
+    const int64_t gx = ((H >= 16 ? 1 : 16 / H) * H + 15) / 16, rows = tile_seq.numel() * gx * 16 * splits;
+    TORCH_CHECK(part_o->numel() >= rows * rank && part_ml->numel() >= rows * 2, "split partial buffers too small");
+    po = part_o->data_ptr<float>();
+    pml = part_ml->data_ptr<float>();
+  }
   ok(dllm_latent_attention(qa.data_ptr(), q.data_ptr(), q.stride(0), f, (int)H, (int)dim, (int)rot, (int)rank, T,
                            cos_sin.data_ptr<float>(), (int)cos_sin.size(1), cache.data_ptr(), bt.data_ptr<int>(),
                            (int)bt.size(1), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                            tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), (float)scale,
-                           out.data_ptr(), stream()),
+                           out.data_ptr(), (int)splits, po, pml, stream()),
      "latent_attention");
 }
 }  // namespace
@@ -1523,7 +1535,10 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("relu2_scale", &relu2_scale);
   m.def("dense_gate", &dense_gate);
   m.def("latent_kv_write", &latent_kv_write);
-  m.def("latent_attention", &latent_attention);
+  m.def("latent_attention", &latent_attention, py::arg("qa"), py::arg("q"), py::arg("dim"), py::arg("rot"),
+        py::arg("positions"), py::arg("cos_sin"), py::arg("cache"), py::arg("block_tables"), py::arg("qstart"),
+        py::arg("qlen"), py::arg("ctx"), py::arg("tile_seq"), py::arg("tile_tok0"), py::arg("scale"), py::arg("out"),
+        py::arg("splits") = 1, py::arg("part_o") = py::none(), py::arg("part_ml") = py::none());
   m.def("encoder_attention", &encoder_attention);
   m.def("embed_ln", &embed_ln);
   m.def("moe_ffn", &moe_ffn, py::arg("x"), py::arg("ids"), py::arg("wts"), py::arg("w13"), py::arg("w2"), py::arg("out"),

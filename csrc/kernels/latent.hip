@@ -14,7 +14,8 @@
 //                     broadcasts, k with an odd row stride: no bank conflicts) -> f32 scores, causal
 //                     mask, online softmax per row (wave reductions);
 //                     phase 2: a lane owns latent dims lane, lane + 64, ... and accumulates p . c.
-//                     Each wave owns 4 of the 16 rows through both phases.
+//                     Each wave owns 4 of the 16 rows through both phases.  Small grids (decode) split
+//                     a row's keys over several workgroups; latent_combine merges their partials.
 // Activations and the cache are bf16 or f32 (template); scores, softmax and sums are f32.
 #include "common.h"
 
@@ -62,7 +63,7 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     const float* __restrict__ cos_sin, int tab_w, const T* __restrict__ cache, const int* __restrict__ bt, int bt_w,
     const int* __restrict__ qstart, const int* __restrict__ qlen, const int* __restrict__ ctx,
     const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, T* __restrict__ out, int KT,
-    int tpe, int kstride, int vec) {
+    int tpe, int kstride, int vec, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
   extern __shared__ float sm[];
   const int entry = blockIdx.y;
   const int s = tile_seq[entry];
@@ -121,8 +122,13 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     for (int i = 0; i < RI; ++i) acc[a][i] = 0.f;
   }
   const int* btr = bt + (long)s * bt_w;
-  for (int k0 = 0; k0 < kmax; k0 += KT) {
-    const int nk = min(KT, kmax - k0);
+  // split over keys (small grids): split z of `splits` walks its share of the key tiles and leaves
+  // unnormalised partials; latent_combine merges them
+  const int ntiles = (kmax + KT - 1) / KT;
+  const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * KT;
+  const int kend = min(kmax, (int)((long)ntiles * (blockIdx.z + 1) / splits) * KT);
+  for (int k0 = kbeg; k0 < kend; k0 += KT) {
+    const int nk = min(KT, kend - k0);
     __syncthreads();   // the previous tile is consumed (and the queries are staged)
     for (int kk = wave; kk < nk; kk += 4) {          // a wave per key row, lanes along the row
       const int kidx = k0 + kk;
@@ -191,6 +197,19 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
       }
     }
   }
+  if (splits > 1) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const long pr = (((long)entry * gridDim.x + blockIdx.x) * LROWS + wave * 4 + a) * splits + blockIdx.z;
+      if (lane == 0) { part_ml[2 * pr] = m[a]; part_ml[2 * pr + 1] = l[a]; }
+#pragma unroll
+      for (int i = 0; i < RI; ++i) {
+        const int c = lane + 64 * i;
+        if (c < rank) part_o[pr * rank + c] = acc[a][i];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
     const int row = row0 + wave * 4 + a;
@@ -203,6 +222,41 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
       const int c = lane + 64 * i;
       if (c < rank) stf(out + ((long)h * Ttot + tok) * rank + c, acc[a][i] * inv);
     }
+  }
+}
+
+// one wave per (entry, row): merge the splits' (max, sum, weighted latent) partials
+template <typename T>
+__global__ void __launch_bounds__(256) latent_combine_kernel(const float* __restrict__ part_o,
+                                                             const float* __restrict__ part_ml, int splits, int gx,
+                                                             int H, int rank, long Ttot, const int* __restrict__ qstart,
+                                                             const int* __restrict__ qlen, const int* __restrict__ tile_seq,
+                                                             const int* __restrict__ tile_tok0, int tpe, long n_rows,
+                                                             T* __restrict__ out) {
+  const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= n_rows) return;
+  const int lane = threadIdx.x & 63;
+  const int rl = (int)(r % LROWS);
+  const long eb = r / LROWS;
+  const int bx = (int)(eb % gx), entry = (int)(eb / gx);
+  const int s = tile_seq[entry];
+  const int n = qlen[s], tok0 = tile_tok0[entry];
+  if (n <= 0 || tok0 >= n) return;
+  const int row = bx * LROWS + rl;
+  if (row >= min(tpe, n - tok0) * H) return;
+  const float* ml = part_ml + 2 * r * splits;
+  float M = -INFINITY;
+  for (int z = 0; z < splits; ++z) M = fmaxf(M, ml[2 * z]);
+  float L = 0.f;
+  for (int z = 0; z < splits; ++z) L += ml[2 * z] == -INFINITY ? 0.f : ml[2 * z + 1] * expf(ml[2 * z] - M);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  const long tok = qstart[s] + tok0 + row / H;
+  const int h = row % H;
+  for (int c = lane; c < rank; c += 64) {
+    float o = 0.f;
+    for (int z = 0; z < splits; ++z)
+      if (ml[2 * z] != -INFINITY) o += part_o[(r * splits + z) * rank + c] * expf(ml[2 * z] - M);
+    stf(out + ((long)h * Ttot + tok) * rank + c, o * inv);
   }
 }
 
@@ -227,7 +281,7 @@ template <typename T>
 int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T* q, long ldq, int H, int dim, int rot,
                   int rank, long Ttot, const float* cos_sin, int tab_w, const T* cache, const int* bt, int bt_w,
                   const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
-                  float scale, T* out, int KT, int tpe, int kstride, int vec) {
+                  float scale, T* out, int KT, int tpe, int kstride, int vec, int splits, float* part_o, float* part_ml) {
 #define LAT(RI)                                                                                                        \
   do {                                                                                                                 \
     if (lds > 48 * 1024)                                                                                               \
@@ -235,10 +289,15 @@ int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T
                           (int)lds);                                                                                   \
     hipLaunchKernelGGL((latent_attention_kernel<T, RI>), g, dim3(256), lds, st, qa, q, ldq, H, dim, rot, rank, Ttot,   \
                        cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT, tpe,   \
-                       kstride, vec);                                                                                  \
+                       kstride, vec, splits, part_o, part_ml);                                                         \
   } while (0)
   if (ri <= 1) LAT(1); else if (ri <= 2) LAT(2); else if (ri <= 4) LAT(4); else LAT(8);
 #undef LAT
+  if (splits > 1) {
+    const long n_rows = (long)g.y * g.x * LROWS;
+    hipLaunchKernelGGL(latent_combine_kernel<T>, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, part_o, part_ml, splits,
+                       (int)g.x, H, rank, Ttot, qstart, qlen, tile_seq, tile_tok0, tpe, n_rows, out);
+  }
   return (int)hipGetLastError();
 }
 }  // namespace
@@ -246,7 +305,8 @@ int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T
 extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, int f32, int H, int dim, int rot, int rank,
                                      long Ttot, const float* cos_sin, int tab_w, const void* cache, const int* bt,
                                      int bt_w, const int* qstart, const int* qlen, const int* ctx, const int* tile_seq,
-                                     const int* tile_tok0, int n_entries, float scale, void* out, hipStream_t st) {
+                                     const int* tile_tok0, int n_entries, float scale, void* out, int splits,
+                                     float* part_o, float* part_ml, hipStream_t st) {
   if (n_entries <= 0 || Ttot <= 0) return 0;
   if (rank < 1 || rank > 512 || rot < 0 || (rot & 1) || rot > tab_w || H < 1) return -1;
   // key rows in LDS: an odd stride for 4-byte reads; when the row length is a multiple of 4 a stride
@@ -258,12 +318,13 @@ extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, in
   const long lds = 4L * (LROWS * Dp + (long)KT * kstride + LROWS * 64);
   if (lds > 150 * 1024) return -2;
   const int tpe = H >= 16 ? 1 : 16 / H;
-  const dim3 g((tpe * H + LROWS - 1) / LROWS, n_entries);
+  if (splits < 1 || (splits > 1 && (!part_o || !part_ml))) return -3;
+  const dim3 g((tpe * H + LROWS - 1) / LROWS, n_entries, splits);
   const int ri = (rank + 63) / 64;
   if (f32)
     return launch_latent<float>(ri, g, lds, st, (const float*)qa, (const float*)q, ldq, H, dim, rot, rank, Ttot, cos_sin,
                                 tab_w, (const float*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale,
-                                (float*)out, KT, tpe, kstride, vec);
+                                (float*)out, KT, tpe, kstride, vec, splits, part_o, part_ml);
   return launch_latent<u16>(ri, g, lds, st, (const u16*)qa, (const u16*)q, ldq, H, dim, rot, rank, Ttot, cos_sin, tab_w,
-                            (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KT, tpe, kstride, vec);
+                            (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KT, tpe, kstride, vec, splits, part_o, part_ml);
 }

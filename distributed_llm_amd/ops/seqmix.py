@@ -92,15 +92,34 @@ def latent_kv_write(ckv, rank, norm_w, eps, positions, cos_sin, slots, cache) ->
     ext.latent_kv_write(ckv, int(rank), norm_w, float(eps), positions, cos_sin, slots, cache)
 
 
+LAT_SPLIT_TARGET = 512     # workgroups a small latent-attention grid is split up to (over keys)
+LAT_SPLIT_MAX = 16
+
+
+def latent_splits(n_entries: int, heads: int) -> int:
+    """Key splits of a latent attention launch: grids with fewer than ``LAT_SPLIT_TARGET`` workgroups
+    (decode steps, short portions) split every row's keys over up to ``LAT_SPLIT_MAX`` workgroups."""
+    gx = ((1 if heads >= 16 else 16 // heads) * heads + LAT_ROWS - 1) // LAT_ROWS
+    return max(1, min(LAT_SPLIT_MAX, LAT_SPLIT_TARGET // max(1, n_entries * gx)))
+
+
 def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx, tile_seq,
-                     tile_tok0, scale) -> torch.Tensor:
+                     tile_tok0, scale, splits: Optional[int] = None) -> torch.Tensor:
     ext = _native(qa)
     if ext is None:
         return ref.latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
                                     scale)
     out = torch.zeros_like(qa)
+    H, n_entries = qa.shape[0], int(tile_seq.numel())
+    sp = latent_splits(n_entries, H) if splits is None else int(splits)
+    po = pml = None
+    if sp > 1:
+        gx = ((1 if H >= 16 else 16 // H) * H + LAT_ROWS - 1) // LAT_ROWS
+        rows = n_entries * gx * LAT_ROWS * sp
+        po = torch.empty(rows * qa.shape[2], dtype=torch.float32, device=qa.device)
+        pml = torch.empty(rows * 2, dtype=torch.float32, device=qa.device)
     ext.latent_attention(qa, q, int(dim), int(rot_dim), positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
-                         tile_seq, tile_tok0, float(scale), out)
+                         tile_seq, tile_tok0, float(scale), out, sp, po, pml)
     return out
 
 

@@ -112,8 +112,9 @@ def test_retention(dt, case, H, d, dv, rot, chunked):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("splits", [1, 3, 16])
 @pytest.mark.parametrize("H,dim,rot,rank", [(8, 64, 32, 64), (3, 16, 8, 40), (20, 32, 16, 128), (1, 8, 64, 512)])
-def test_latent_attention(dt, case, H, dim, rot, rank):
+def test_latent_attention(dt, case, H, dim, rot, rank, splits):
     torch.manual_seed(3)
     qlens, starts = case
     T, qstart, qlen, ctx, rows, pos = batch(qlens, starts)
@@ -143,7 +144,7 @@ def test_latent_attention(dt, case, H, dim, rot, rank):
     meta = AttnMeta(slots=None, block_tables=perm, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
                     last_idx=None, host_qlen=qlens)
     ts, tt = meta.latent_tiles(H, DEV)
-    o1 = seqmix.latent_attention(qa, q, dim, rot, pos, table, cache2, perm, qstart, qlen, ctx, ts, tt, 0.2)
+    o1 = seqmix.latent_attention(qa, q, dim, rot, pos, table, cache2, perm, qstart, qlen, ctx, ts, tt, 0.2, splits=splits)
     o2 = ref.latent_attention(qa, q, dim, rot, pos, table, cache2, perm, qstart, qlen, ctx, 0.2)
     torch.testing.assert_close(o1.float(), o2.float(), **tol(dt))
 
