@@ -41,7 +41,7 @@ from .configs import HybridConfig, LayerSpec, MixerSpec, MoESpec
 def _mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """x @ w.T: the framework's tuned GEMM where it takes the shape, else the vendor GEMM."""
     if (x.is_cuda and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1
-            and x.shape[1] % 64 == 0 and w.shape[0] % 16 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and x.shape[1] % 64 == 0 and w.shape[0] % 64 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
             and w.is_contiguous()):
         return ops.linear(x, w)
     return F.linear(x, w)
@@ -270,7 +270,10 @@ class HybridModel:
         return _mm(o.transpose(0, 1).reshape(T, H * m.vdim), L["o"])
 
     def _experts(self, L, f: MoESpec, x):
-        if x.is_cuda and x.dtype == torch.bfloat16:
+        if f.experts > 64 or f.top > 8:      # beyond the router kernels' register budget: library top-k
+            val, ids = torch.topk(torch.softmax(F.linear(x.float(), L["router"].float()), -1), f.top, -1)
+            ids, w = ids.to(torch.int32), val / (val.sum(-1, keepdim=True) + 1e-20)
+        elif x.is_cuda and x.dtype == torch.bfloat16:
             ids, w = ops.moe_router(x, L["router"], f.top)      # f32 logits, softmax over the chosen = s / sum s
         else:
             ids, w = ops.moe_gate(F.linear(x.float(), L["router"].float()), f.top)
@@ -296,7 +299,10 @@ class HybridModel:
         if scatter is not None:
             ops.scatter_pairs(*scatter)
         if self.dtype == torch.bfloat16:
-            xl = ops.embedding(input_ids, self.embed)
+            if cfg.hidden % 8 == 0:
+                xl = ops.embedding(input_ids, self.embed)
+            else:      # the gather kernel moves 16-byte vectors
+                xl = self.embed.index_select(0, input_ids.long())
             x = xl.float()
         else:
             x = self.embed.index_select(0, input_ids.long())
@@ -326,11 +332,21 @@ class HybridModel:
     def logits_f32(self, hidden: torch.Tensor) -> torch.Tensor:
         return _mm(hidden, self.lm_head).float() * self.cfg.logit_scale
 
+    def _sampler_logits(self, hidden: torch.Tensor) -> torch.Tensor:
+        """bf16 logits [S, vocab] whose rows start 16-byte aligned (the sampler kernels read vectors)."""
+        lg = self.logits(hidden)
+        V = lg.shape[1]
+        if V % 8 == 0 or not lg.is_cuda:
+            return lg.to(torch.bfloat16)
+        buf = torch.zeros((lg.shape[0], (V + 7) // 8 * 8), dtype=torch.bfloat16, device=lg.device)
+        buf[:, :V].copy_(lg)
+        return buf[:, :V]
+
     def greedy(self, hidden: torch.Tensor) -> torch.Tensor:
-        return ops.argmax(self.logits(hidden).to(torch.bfloat16) if hidden.is_cuda else self.logits(hidden))
+        return ops.argmax(self._sampler_logits(hidden))
 
     def sample(self, hidden, temperature, top_p, top_k, seed, out):
-        return ops.sample_rows(self.logits(hidden).to(torch.bfloat16), temperature, top_p, top_k, seed, out=out)
+        return ops.sample_rows(self._sampler_logits(hidden), temperature, top_p, top_k, seed, out=out)
 
     def topk_candidates(self, hidden: torch.Tensor, k: int):
         v, i = torch.topk(self.logits(hidden).float(), min(k, self.cfg.vocab), dim=-1)

@@ -65,6 +65,14 @@ def selective_scan(xc, dt_raw, dt_bias, A, dbc, dt_rank, D, xz, ssm_state, conv_
     return out
 
 
+def retention_step_lds(dim: int, vdim: int) -> int:
+    """LDS bytes of the token-by-token retention kernel (csrc/kernels/seqmix.hip dllm_retention_lds)."""
+    lj = 1
+    while lj < vdim and lj < 64:
+        lj <<= 1
+    return 4 * (dim * vdim + 8 * (2 * dim + 2 * vdim) + 2 * (256 // lj) * vdim)
+
+
 RETENTION_CHUNK_MIN = 4    # average new tokens per sequence from which the chunked kernel runs
 
 
@@ -79,6 +87,8 @@ def retention(qkvg, heads, dim, vdim, cos_sin, rot_dims, decay, state, eps, posi
     out = torch.zeros((qkvg.shape[0], heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
     if chunked is None:
         chunked = qkvg.shape[0] >= RETENTION_CHUNK_MIN * qstart.numel()
+    if not chunked and retention_step_lds(dim, vdim) > 150 * 1024:
+        chunked = True      # the token-by-token kernel keeps the whole [dim, vdim] state in LDS
     raw = torch.empty((qkvg.shape[0], heads, vdim), dtype=torch.float32, device=qkvg.device) if chunked else None
     ext.retention(qkvg, int(heads), int(dim), int(vdim), cos_sin, int(rot_dims), decay, state, float(eps), positions,
                   qstart, qlen, ctx, rows, out, raw)

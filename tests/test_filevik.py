@@ -157,6 +157,8 @@ SINGLE = {
     "latent": [latent()], "latent-many-heads": [latent(heads=18, dim=4, rot_dim=2, vdim=3, kv_rank=70, q_rank=9)],
     "experts": [dict(mamba(), mlp=moe())], "experts-no-shared": [dict(reten(), mlp=moe(experts=6, top=3, shared=0))],
     "experts-all": [dict(latent(), mlp=moe(experts=2, top=2, scale=1.0))],
+    "experts-many": [dict(mamba(), mlp=moe(experts=70, top=9, ff=3, shared=5))],
+    "retention-large-state": [reten(heads=1, dim=96, vdim=200, decay=(0.98,), rot=32)],
 }
 
 
@@ -295,6 +297,30 @@ def test_greedy_generation(full_model, device):
     for p, o in zip(prompts, outs):
         assert o.error is None
         assert o.token_ids == orc.greedy(cfg, W, p, 12)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_unaligned_sizes(tmp_path, device, dtype):
+    """Width, vocabulary and inner sizes that no 16-byte vector or 64-wide tile divides: every kernel's
+    scalar tail and the library-GEMM routes; generation samples from an unaligned vocabulary."""
+    layers = [dict(mamba(inner=14, state=3, dt_rank=1, conv=2), mlp=moe(experts=3, top=2, ff=5, shared=7)),
+              dict(reten(heads=1, dim=6, vdim=5, decay=(0.93,), rot=2), mlp=None),
+              dict(latent(heads=5, dim=3, rot_dim=2, vdim=7, kv_rank=9, q_rank=11), mlp=moe(experts=2, top=1, ff=3, shared=0))]
+    if dtype == torch.bfloat16:
+        for L in layers:
+            if L["mlp"]:
+                L["mlp"]["router"]["top"] = L["mlp"]["router"]["experts"]
+    cfg = make_cfg(layers, width=20, vocab=37, logit_scale=1.0)
+    W = make_weights(cfg, seed=6)
+    eng = engine(write_model(tmp_path / "m", cfg, W), device, dtype)
+    t = toks(30, vocab=37, seed=3)
+    want = orc.forward(cfg, W, t)
+    got = [eng.feed([("a", t[:21], list(range(21)))])] + [eng.feed([("a", t[i:i + 1], [0])]) for i in range(21, 30)]
+    close(torch.cat(got), want, dtype, "unaligned")
+    if dtype == torch.float32:
+        out = eng.generate([t[:7]], SamplingParams(max_new_tokens=5, temperature=0.0, ignore_eos=True))[0]
+        assert out.token_ids == orc.greedy(cfg, W, t[:7], 5)
 
 
 def test_registry_reads_config(full_model):
