@@ -56,6 +56,23 @@ __global__ void __launch_bounds__(64) latent_kv_write_kernel(const T* __restrict
 
 constexpr int LROWS = 16;
 
+// one cache row -> f32 in LDS, lanes along the row (bf16 rows of even length move 4 bytes per lane)
+__device__ __forceinline__ void stage_row(const float* src, float* dst, int Dp, int lane) {
+  for (int c = lane; c < Dp; c += 64) dst[c] = src[c];
+}
+__device__ __forceinline__ void stage_row(const u16* src, float* dst, int Dp, int lane) {
+  if ((Dp & 1) == 0) {
+    const uint32_t* s2 = reinterpret_cast<const uint32_t*>(src);
+    for (int c = lane; c < (Dp >> 1); c += 64) {
+      const uint32_t w = s2[c];
+      dst[2 * c] = __uint_as_float(w << 16);
+      dst[2 * c + 1] = __uint_as_float(w & 0xffff0000u);
+    }
+  } else {
+    for (int c = lane; c < Dp; c += 64) dst[c] = bf2f(src[c]);
+  }
+}
+
 // RI: latent dims per lane in phase 2 (rank <= 64 RI)
 template <typename T, int RI>
 __global__ void __launch_bounds__(256) latent_attention_kernel(
@@ -130,11 +147,14 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     const int nk = min(KT, kend - k0);
     __syncthreads();   // the previous tile is consumed (and the queries are staged)
+    // the tile's pages: read once, so the row loads below do not each wait for a block-table entry
+    const int pg0 = k0 >> 4, npg = ((k0 + nk - 1) >> 4) - pg0 + 1;
+    const int pg = lane < npg ? btr[pg0 + lane] : 0;
+#pragma unroll 4
     for (int kk = wave; kk < nk; kk += 4) {          // a wave per key row, lanes along the row
       const int kidx = k0 + kk;
-      const T* src = cache + ((long)btr[kidx >> 4] * 16 + (kidx & 15)) * Dp;
-      float* dst = ksh + kk * kstride;
-      for (int c = lane; c < Dp; c += 64) dst[c] = ldf(src + c);
+      const long page = __shfl(pg, (kidx >> 4) - pg0);
+      stage_row(cache + (page * 16 + (kidx & 15)) * Dp, ksh + kk * kstride, Dp, lane);
     }
     __syncthreads();
     // phase 1: lane = key
@@ -143,7 +163,7 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
       const float* kr = ksh + lane * kstride;
       const float* qr = qsh + (wave * 4) * Dp;
       if (vec) {          // 16-byte LDS reads: rows are 16-byte aligned, kstride / 4 is odd (no bank conflicts)
-#pragma unroll 2
+#pragma unroll 8
         for (int c = 0; c < Dp; c += 4) {
           const float4 kv = *reinterpret_cast<const float4*>(kr + c);
 #pragma unroll
@@ -182,6 +202,7 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
     for (int a = 0; a < 4; ++a)
 #pragma unroll
       for (int i = 0; i < RI; ++i) acc[a][i] *= alpha[a];
+#pragma unroll 4
     for (int kk = 0; kk < nk; ++kk) {
       float kv[RI];
 #pragma unroll

@@ -365,7 +365,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restric
       if (u0 <= t) {
         const float* q = Qs + t * dp;
         const float* k = Ks + u0 * dp;
-#pragma unroll 4
+#pragma unroll 8
         for (int i = 0; i < d; ++i) {
           const float qv = q[i];
 #pragma unroll
@@ -384,7 +384,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restric
       const int t = tid >> 3, j0 = (tid & 7) * 4;
       const float* q = Qs + t * dp;
       float o4[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+#pragma unroll 8
       for (int i = 0; i < d; ++i) {
         const float qv = q[i];
         const float4 sv = *reinterpret_cast<const float4*>(S + i * RC_V + j0);
@@ -414,6 +414,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restric
         float acc[16];
 #pragma unroll
         for (int x = 0; x < 16; ++x) acc[x] = gn * S[i * RC_V + jb + x];
+#pragma unroll 4
         for (int u = 0; u < nt; ++u) {
           const float kv = gp[nt - 1 - u] * Ks[u * dp + i];
           const float* v = Vs + u * RC_V + jb;
