@@ -232,6 +232,9 @@ class LLMEngine:
             kv_cache_gb = min(float(kv_cache_gb), max(0.5, free / 2**30 - KV_RESERVE_GB))
         self.kv_cache_gb = float(kv_cache_gb)
         self.num_blocks = max(int(kv_cache_gb * 2**30) // per_block, self.max_blocks + 8)
+        if own and m.block_bytes(BS) == 0:
+            # nothing is paged (recurrent layers only): blocks are bookkeeping, every row may run full length
+            self.num_blocks = self.max_num_seqs * self.max_blocks + 8
         if num_kv_blocks is not None:
             self.num_blocks = int(num_kv_blocks)
         if own:
