@@ -305,9 +305,12 @@ int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T
                   float scale, T* out, int KT, int tpe, int kstride, int vec, int splits, float* part_o, float* part_ml) {
 #define LAT(RI)                                                                                                        \
   do {                                                                                                                 \
-    if (lds > 48 * 1024)                                                                                               \
+    static long have_ = 48 * 1024; /* raised once per size: no attribute call inside a later stream capture */        \
+    if (lds > have_) {                                                                                                 \
       hipFuncSetAttribute((const void*)latent_attention_kernel<T, RI>, hipFuncAttributeMaxDynamicSharedMemorySize,    \
                           (int)lds);                                                                                   \
+      have_ = lds;                                                                                                     \
+    }                                                                                                                  \
     hipLaunchKernelGGL((latent_attention_kernel<T, RI>), g, dim3(256), lds, st, qa, q, ldq, H, dim, rot, rank, Ttot,   \
                        cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT, tpe,   \
                        kstride, vec, splits, part_o, part_ml);                                                         \

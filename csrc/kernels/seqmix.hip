@@ -484,6 +484,17 @@ __global__ void __launch_bounds__(256) dense_gate_kernel(const int* __restrict__
 
 }  // namespace
 
+// Raise a kernel's dynamic-LDS limit when a launch needs more than it has been given so far (once per
+// size: a later launch inside a stream capture then makes no attribute call).
+#define ENSURE_LDS(kernel, bytes)                                                                          \
+  do {                                                                                                     \
+    static long have_ = 48 * 1024;                                                                         \
+    if ((bytes) > have_) {                                                                                 \
+      hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(bytes)); \
+      have_ = (bytes);                                                                                     \
+    }                                                                                                      \
+  } while (0)
+
 #define BY_T(f32, call_u16, call_f32) \
   if (f32) { call_f32; } else { call_u16; }
 
@@ -570,11 +581,11 @@ extern "C" int dllm_retention(const void* qkvg, long ld, int f32, int H, int d, 
   while (lj < dv && lj < 64) lj <<= 1;
   const dim3 g(H, S);
   if (f32) {
-    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    ENSURE_LDS(retention_kernel<float>, lds);
     hipLaunchKernelGGL(retention_kernel<float>, g, dim3(256), lds, st, (const float*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
                        decay, state, eps, qstart, qlen, ctx, rows, (float*)out, lj);
   } else {
-    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    ENSURE_LDS(retention_kernel<u16>, lds);
     hipLaunchKernelGGL(retention_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
                        decay, state, eps, qstart, qlen, ctx, rows, (u16*)out, lj);
   }
@@ -598,13 +609,13 @@ extern "C" int dllm_retention_chunked(const void* qkvg, long ld, int f32, int H,
   const long rows_total = T * H;
   const dim3 gf((unsigned)((rows_total + 3) / 4));
   if (f32) {
-    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_chunk_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    ENSURE_LDS(retention_chunk_kernel<float>, lds);
     hipLaunchKernelGGL(retention_chunk_kernel<float>, g, dim3(256), lds, st, (const float*)qkvg, ld, H, d, dv, cos_sin, tab_w,
                        rot, decay, state, qstart, qlen, ctx, rows, raw);
     hipLaunchKernelGGL(retention_finish_kernel<float>, gf, dim3(256), 0, st, raw, (const float*)qkvg, ld, H, d, dv, eps, qstart,
                        qlen, S, (float*)out, rows_total);
   } else {
-    if (lds > 48 * 1024) hipFuncSetAttribute((const void*)retention_chunk_kernel<u16>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    ENSURE_LDS(retention_chunk_kernel<u16>, lds);
     hipLaunchKernelGGL(retention_chunk_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
                        decay, state, qstart, qlen, ctx, rows, raw);
     hipLaunchKernelGGL(retention_finish_kernel<u16>, gf, dim3(256), 0, st, raw, (const u16*)qkvg, ld, H, d, dv, eps, qstart, qlen,
