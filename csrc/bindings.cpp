@@ -67,7 +67,7 @@ int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, 
                          void*, int, hipStream_t);
 int dllm_latent_attention(const void*, const void*, long, int, int, int, int, int, long, const float*, int, const void*,
                           const int*, int, const int*, const int*, const int*, const int*, const int*, int, float, void*,
-                          int, float*, float*, hipStream_t);
+                          int, float*, float*, int, hipStream_t);
 int dllm_car_alloc(long, void**);
 int dllm_car_get_handle(void*, char*);
 int dllm_car_handle_size();
@@ -1484,7 +1484,7 @@ void latent_kv_write(torch::Tensor ckv, int64_t rank, torch::Tensor w, double ep
 void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t rot, torch::Tensor pos, torch::Tensor cos_sin,
                       torch::Tensor cache, torch::Tensor bt, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
                       torch::Tensor tile_seq, torch::Tensor tile_tok0, double scale, torch::Tensor out, int64_t splits,
-                      c10::optional<torch::Tensor> part_o, c10::optional<torch::Tensor> part_ml) {
+                      c10::optional<torch::Tensor> part_o, c10::optional<torch::Tensor> part_ml, bool mfma) {
   const bool f = act_f32(qa, "qa");
   TORCH_CHECK(qa.dim() == 3 && qa.is_contiguous(), "qa [H, T, rank] contiguous");
   const int64_t H = qa.size(0), T = qa.size(1), rank = qa.size(2);
@@ -1519,7 +1519,7 @@ void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t ro
                            cos_sin.data_ptr<float>(), (int)cos_sin.size(1), cache.data_ptr(), bt.data_ptr<int>(),
                            (int)bt.size(1), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                            tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), (float)scale,
-                           out.data_ptr(), (int)splits, po, pml, stream()),
+                           out.data_ptr(), (int)splits, po, pml, mfma ? 1 : 0, stream()),
      "latent_attention");
 }
 }  // namespace
@@ -1538,7 +1538,7 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("latent_attention", &latent_attention, py::arg("qa"), py::arg("q"), py::arg("dim"), py::arg("rot"),
         py::arg("positions"), py::arg("cos_sin"), py::arg("cache"), py::arg("block_tables"), py::arg("qstart"),
         py::arg("qlen"), py::arg("ctx"), py::arg("tile_seq"), py::arg("tile_tok0"), py::arg("scale"), py::arg("out"),
-        py::arg("splits") = 1, py::arg("part_o") = py::none(), py::arg("part_ml") = py::none());
+        py::arg("splits") = 1, py::arg("part_o") = py::none(), py::arg("part_ml") = py::none(), py::arg("mfma") = true);
   m.def("encoder_attention", &encoder_attention);
   m.def("embed_ln", &embed_ln);
   m.def("moe_ffn", &moe_ffn, py::arg("x"), py::arg("ids"), py::arg("wts"), py::arg("w13"), py::arg("w2"), py::arg("out"),

@@ -246,6 +246,245 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
   }
 }
 
+// ---------------------------------------------------------------- bf16 models: matrix-core form
+// Same row blocks, key tiles, causal mask, online softmax and key splits as above, with both products
+// on v_mfma_f32_16x16x32_bf16 (operands bf16 from the cache, f32 accumulation):
+//   scores   S[16 rows x 16 keys] per wave (wave w: keys 16w..16w+15 of the tile): A = query rows
+//            (LDS, bf16, the rotation applied while staging, the score scale applied to the f32 sums),
+//            B = key rows (LDS, row-major copy of the tile);
+//   softmax  in the accumulator layout (a lane holds rows 4g..4g+3 of one key): row maxima by DPP
+//            over the 16 lanes of a row group, then across the waves through LDS; a lane keeps a
+//            partial row sum of its own keys until the end;
+//   weights  written to LDS as bf16 hi + lo parts (p = hi + lo to 2^-17), so the second product sees
+//            f32 weights to 16 bits of mantissa through two MFMAs;
+//   output   O[16 rows x rank]: wave w owns latent column blocks w, w + 4, ...; A = weights (hi, lo),
+//            B = a TRANSPOSED copy of the tile's latent part in LDS ([dim][key], written while
+//            staging), because the product contracts over keys and an operand holds 8 consecutive
+//            contraction indices per lane.
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));
+  return v;
+}
+__device__ __forceinline__ float row16_add(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+
+struct MfmaLds { int Dpad, qstr, ktstr, pstr, RB; long bytes; };
+static inline MfmaLds mfma_lds(int rank, int rot, int KT) {
+  MfmaLds L;
+  L.Dpad = (rank + rot + 31) & ~31;
+  L.qstr = L.Dpad + 8;
+  L.ktstr = KT + 2;
+  L.pstr = KT + 8;
+  L.RB = (rank + 15) / 16;
+  L.bytes = 2L * (LROWS * L.qstr + (long)KT * L.qstr + (long)L.RB * 16 * L.ktstr + 2L * LROWS * L.pstr) + 4L * 4 * LROWS;
+  return L;
+}
+
+template <int CB>
+__global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
+    const u16* __restrict__ qa, const u16* __restrict__ q, long ldq, int H, int dim, int rot, int rank, long Ttot,
+    const float* __restrict__ cos_sin, int tab_w, const u16* __restrict__ cache, const int* __restrict__ bt, int bt_w,
+    const int* __restrict__ qstart, const int* __restrict__ qlen, const int* __restrict__ ctx,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, u16* __restrict__ out, int KT,
+    int tpe, int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int Dpad, int qstr, int ktstr,
+    int pstr, int RB) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
+  const int entry = blockIdx.y;
+  const int s = tile_seq[entry];
+  const int n = qlen[s];
+  if (n <= 0) return;
+  const int tok0 = tile_tok0[entry];
+  if (tok0 >= n) return;
+  const int ntok = min(tpe, n - tok0);
+  const int nrows = ntok * H;
+  const int row0 = blockIdx.x * LROWS;
+  if (row0 >= nrows) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  const int Dp = rank + rot;
+  u16* qsh = reinterpret_cast<u16*>(smraw);             // [16][qstr]
+  u16* ksh = qsh + LROWS * qstr;                        // [KT][qstr]
+  u16* ktr = ksh + KT * qstr;                           // [RB * 16][ktstr]: latent part transposed
+  u16* phi = ktr + RB * 16 * ktstr;                     // [16][pstr]
+  u16* plo = phi + LROWS * pstr;
+  float* wred = reinterpret_cast<float*>(plo + LROWS * pstr);   // [4][16]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, g = lane >> 4;
+  const int half = rot >> 1;
+  for (int e = tid; e < LROWS * Dpad; e += 256) {
+    const int rr = e / Dpad, c = e - rr * Dpad, row = row0 + rr;
+    float v = 0.f;
+    if (row < nrows && c < Dp) {
+      const int tl = tok0 + row / H, h = row % H;
+      const long tok = q0 + tl;
+      if (c < rank) {
+        v = bf2f(qa[((long)h * Ttot + tok) * rank + c]);
+      } else {
+        const int i = (c - rank) >> 1;
+        const u16* qr = q + tok * ldq + (long)h * (dim + rot) + dim + 2 * i;
+        const float u = bf2f(qr[0]), w = bf2f(qr[1]);
+        const float* cs = cos_sin + (long)(p0 + tl) * tab_w;
+        v = ((c - rank) & 1) ? w * cs[i] + u * cs[half + i] : u * cs[i] - w * cs[half + i];
+      }
+    }
+    qsh[rr * qstr + c] = f2bf(v);
+  }
+  // zero what no staging pass writes: the transposed tile's padded rows and the key rows' padded dims
+  for (int e = tid; e < RB * 16 * ktstr; e += 256) ktr[e] = 0;
+  for (int e = tid; e < KT * qstr; e += 256) ksh[e] = 0;
+  const int last_row = min(row0 + LROWS, nrows) - 1;
+  const int kmax = p0 + tok0 + last_row / H + 1;
+  int rpos[4];
+  bool rok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = row0 + 4 * g + i;
+    rok[i] = row < nrows;
+    rpos[i] = p0 + tok0 + (rok[i] ? row / H : 0);
+  }
+  float m[4], l[4];
+  f32x4 acc[CB];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -INFINITY; l[i] = 0.f; }
+#pragma unroll
+  for (int j = 0; j < CB; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int* btr = bt + (long)s * bt_w;
+  const int ntiles = (kmax + KT - 1) / KT;
+  const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * KT;
+  const int kend = min(kmax, (int)((long)ntiles * (blockIdx.z + 1) / splits) * KT);
+  const int NKB = KT >> 4;
+  for (int k0 = kbeg; k0 < kend; k0 += KT) {
+    const int nk = min(KT, kend - k0);
+    __syncthreads();
+    const int pg0 = k0 >> 4, npg = ((k0 + nk - 1) >> 4) - pg0 + 1;
+    const int pg = lane < npg ? btr[pg0 + lane] : 0;
+    for (int kk = wave; kk < KT; kk += 4) {        // a wave per key row; rows past the tile's end are zeros
+      const int kidx = k0 + kk;
+      const bool live = kk < nk;
+      const long page = __shfl(pg, live ? (kidx >> 4) - pg0 : 0);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(cache + (page * 16 + (kidx & 15)) * Dp);
+      for (int c2 = lane; c2 < (Dp >> 1); c2 += 64) {
+        const uint32_t w = live ? src[c2] : 0u;
+        *reinterpret_cast<uint32_t*>(ksh + kk * qstr + 2 * c2) = w;
+        if (2 * c2 < rank) {
+          ktr[(2 * c2) * ktstr + kk] = (u16)(w & 0xffffu);
+          ktr[(2 * c2 + 1) * ktstr + kk] = (u16)(w >> 16);
+        }
+      }
+    }
+    __syncthreads();
+    // scores of this wave's 16 keys
+    f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+    if (wave < NKB) {
+      const u16* ap = qsh + lr * qstr + 8 * g;
+      const u16* bp = ksh + (16 * wave + lr) * qstr + 8 * g;
+      for (int st = 0; st < Dpad; st += 32) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ap + st));
+        const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + st));
+        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, sacc, 0, 0, 0);
+      }
+    }
+    const int kidx = k0 + 16 * wave + lr;
+    float sv[4];
+    bool vis[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      vis[i] = wave < NKB && kidx < kend && rok[i] && kidx <= rpos[i];
+      sv[i] = vis[i] ? sacc[i] * scale : -INFINITY;
+      const float wm = row16_max(sv[i]);
+      if (lr == 0) wred[wave * LROWS + 4 * g + i] = wm;
+    }
+    __syncthreads();
+    float alpha[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * g + i;
+      const float tm = fmaxf(fmaxf(wred[r], wred[LROWS + r]), fmaxf(wred[2 * LROWS + r], wred[3 * LROWS + r]));
+      const float mn = fmaxf(m[i], tm);
+      float p = 0.f;
+      alpha[i] = 1.f;
+      if (mn != -INFINITY) {
+        p = vis[i] ? expf(sv[i] - mn) : 0.f;
+        alpha[i] = expf(m[i] - mn);
+        m[i] = mn;
+      }
+      l[i] = l[i] * alpha[i] + p;
+      if (wave < NKB) {
+        const u16 hi = f2bf(p);
+        phi[r * pstr + 16 * wave + lr] = hi;
+        plo[r * pstr + 16 * wave + lr] = f2bf(p - bf2f(hi));
+      }
+    }
+    __syncthreads();
+    // weighted latents of this wave's column blocks
+#pragma unroll
+    for (int j = 0; j < CB; ++j) {
+      const int cb = wave + 4 * j;
+      if (cb < RB) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] *= alpha[i];
+        const u16* bp = ktr + (cb * 16 + lr) * ktstr + 8 * g;
+        for (int ks = 0; ks < KT; ks += 32) {
+          const bf16x8 ah = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(phi + lr * pstr + ks + 8 * g));
+          const bf16x8 al = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(plo + lr * pstr + ks + 8 * g));
+          const uint32_t* b32 = reinterpret_cast<const uint32_t*>(bp + ks);
+          const uint4 bw = make_uint4(b32[0], b32[1], b32[2], b32[3]);
+          const bf16x8 b = __builtin_bit_cast(bf16x8, bw);
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, b, acc[j], 0, 0, 0);
+          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, b, acc[j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // row sums: over the 16 lanes of a row group, then over the waves
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float t = row16_add(l[i]);
+    if (lr == 0) wred[wave * LROWS + 4 * g + i] = t;
+  }
+  __syncthreads();
+  float lt[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * g + i;
+    lt[i] = wred[r] + wred[LROWS + r] + wred[2 * LROWS + r] + wred[3 * LROWS + r];
+  }
+  if (splits > 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const long pr = (((long)entry * gridDim.x + blockIdx.x) * LROWS + 4 * g + i) * splits + blockIdx.z;
+      if (wave == 0 && lr == 0) { part_ml[2 * pr] = m[i]; part_ml[2 * pr + 1] = lt[i]; }
+#pragma unroll
+      for (int j = 0; j < CB; ++j) {
+        const int c = (wave + 4 * j) * 16 + lr;
+        if (wave + 4 * j < RB && c < rank) part_o[pr * rank + c] = acc[j][i];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = row0 + 4 * g + i;
+    if (row >= nrows) continue;
+    const long tok = q0 + tok0 + row / H;
+    const int h = row % H;
+    const float inv = lt[i] > 0.f ? 1.f / lt[i] : 0.f;
+#pragma unroll
+    for (int j = 0; j < CB; ++j) {
+      const int c = (wave + 4 * j) * 16 + lr;
+      if (wave + 4 * j < RB && c < rank) out[((long)h * Ttot + tok) * rank + c] = f2bf(acc[j][i] * inv);
+    }
+  }
+}
+
 // one wave per (entry, row): merge the splits' (max, sum, weighted latent) partials
 template <typename T>
 __global__ void __launch_bounds__(256) latent_combine_kernel(const float* __restrict__ part_o,
@@ -326,13 +565,58 @@ int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T
 }
 }  // namespace
 
+namespace {
+int launch_latent_mfma(dim3 g, hipStream_t st, const u16* qa, const u16* q, long ldq, int H, int dim, int rot, int rank,
+                       long Ttot, const float* cos_sin, int tab_w, const u16* cache, const int* bt, int bt_w,
+                       const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
+                       float scale, u16* out, int KT, int tpe, int splits, float* part_o, float* part_ml) {
+  const MfmaLds L = mfma_lds(rank, rot, KT);
+  const int cbs = (L.RB + 3) / 4;
+#define LATM(CB)                                                                                                       \
+  do {                                                                                                                 \
+    static long have_ = 48 * 1024;                                                                                     \
+    if (L.bytes > have_) {                                                                                             \
+      hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<CB>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                          (int)L.bytes);                                                                               \
+      have_ = L.bytes;                                                                                                 \
+    }                                                                                                                  \
+    hipLaunchKernelGGL((latent_attention_mfma_kernel<CB>), g, dim3(256), L.bytes, st, qa, q, ldq, H, dim, rot, rank,   \
+                       Ttot, cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT,  \
+                       tpe, splits, part_o, part_ml, L.Dpad, L.qstr, L.ktstr, L.pstr, L.RB);                           \
+  } while (0)
+  if (cbs <= 1) LATM(1); else if (cbs <= 2) LATM(2); else if (cbs <= 4) LATM(4); else LATM(8);
+#undef LATM
+  if (splits > 1) {
+    const long n_rows = (long)g.y * g.x * LROWS;
+    hipLaunchKernelGGL(latent_combine_kernel<u16>, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, part_o, part_ml,
+                       splits, (int)g.x, H, rank, Ttot, qstart, qlen, tile_seq, tile_tok0, tpe, n_rows, out);
+  }
+  return (int)hipGetLastError();
+}
+}  // namespace
+
+// 1 when the matrix-core kernel takes this shape (bf16, even widths, a 32-key tile fits the LDS)
+extern "C" int dllm_latent_mfma_ok(int rank, int rot) {
+  if ((rank & 1) || (rot & 1) || rank < 2 || rank > 512) return 0;
+  return mfma_lds(rank, rot, 32).bytes <= 150 * 1024;
+}
+
 extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, int f32, int H, int dim, int rot, int rank,
                                      long Ttot, const float* cos_sin, int tab_w, const void* cache, const int* bt,
                                      int bt_w, const int* qstart, const int* qlen, const int* ctx, const int* tile_seq,
                                      const int* tile_tok0, int n_entries, float scale, void* out, int splits,
-                                     float* part_o, float* part_ml, hipStream_t st) {
+                                     float* part_o, float* part_ml, int mfma, hipStream_t st) {
   if (n_entries <= 0 || Ttot <= 0) return 0;
   if (rank < 1 || rank > 512 || rot < 0 || (rot & 1) || rot > tab_w || H < 1) return -1;
+  if (splits < 1 || (splits > 1 && (!part_o || !part_ml))) return -3;
+  if (mfma && !f32 && dllm_latent_mfma_ok(rank, rot)) {
+    const int KTm = mfma_lds(rank, rot, 64).bytes <= 150 * 1024 ? 64 : 32;
+    const int tpe_m = H >= 16 ? 1 : 16 / H;
+    const dim3 gm((tpe_m * H + LROWS - 1) / LROWS, n_entries, splits);
+    return launch_latent_mfma(gm, st, (const u16*)qa, (const u16*)q, ldq, H, dim, rot, rank, Ttot, cos_sin, tab_w,
+                              (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KTm,
+                              tpe_m, splits, part_o, part_ml);
+  }
   // key rows in LDS: an odd stride for 4-byte reads; when the row length is a multiple of 4 a stride
   // that is 4 x odd, so a lane's 16-byte reads are aligned and spread over all banks
   const int Dp = rank + rot, vec = (Dp & 3) == 0;

@@ -12,6 +12,7 @@ sequence whose first new position is 0 starts from a zero state, so a re-used sl
 """
 from __future__ import annotations
 
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -114,7 +115,9 @@ def latent_splits(n_entries: int, heads: int) -> int:
 
 
 def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx, tile_seq,
-                     tile_tok0, scale, splits: Optional[int] = None) -> torch.Tensor:
+                     tile_tok0, scale, splits: Optional[int] = None, mfma: Optional[bool] = None) -> torch.Tensor:
+    """``mfma`` (GPU, bf16): the matrix-core kernel (default where the shape fits it;
+    ``DLLM_LATENT_MFMA=0`` or ``mfma=False`` keeps the vector-ALU kernel that f32 models run)."""
     ext = _native(qa)
     if ext is None:
         return ref.latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
@@ -128,8 +131,10 @@ def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_table
         rows = n_entries * gx * LAT_ROWS * sp
         po = torch.empty(rows * qa.shape[2], dtype=torch.float32, device=qa.device)
         pml = torch.empty(rows * 2, dtype=torch.float32, device=qa.device)
+    if mfma is None:
+        mfma = os.environ.get("DLLM_LATENT_MFMA", "1") == "1"
     ext.latent_attention(qa, q, int(dim), int(rot_dim), positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
-                         tile_seq, tile_tok0, float(scale), out, sp, po, pml)
+                         tile_seq, tile_tok0, float(scale), out, sp, po, pml, bool(mfma))
     return out
 
 
