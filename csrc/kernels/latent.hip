@@ -258,9 +258,9 @@ __global__ void __launch_bounds__(256) latent_attention_kernel(
 //   weights  written to LDS as bf16 hi + lo parts (p = hi + lo to 2^-17), so the second product sees
 //            f32 weights to 16 bits of mantissa through two MFMAs;
 //   output   O[16 rows x rank]: wave w owns latent column blocks w, w + 4, ...; A = weights (hi, lo),
-//            B = a TRANSPOSED copy of the tile's latent part in LDS ([dim][key], written while
-//            staging), because the product contracts over keys and an operand holds 8 consecutive
-//            contraction indices per lane.
+//            B = a TRANSPOSED copy of the tile's latent part in LDS ([dim][key], made from the
+//            row-major tile by a second pass), because the product contracts over keys and an operand
+//            holds 8 consecutive contraction indices per lane.
 __device__ __forceinline__ float row16_max(float v) {
   v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));
   v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));
@@ -281,19 +281,19 @@ static inline MfmaLds mfma_lds(int rank, int rot, int KT) {
   MfmaLds L;
   L.Dpad = (rank + rot + 31) & ~31;
   L.qstr = L.Dpad + 8;
-  L.ktstr = KT + 2;
+  L.ktstr = KT + 8;
   L.pstr = KT + 8;
   L.RB = (rank + 15) / 16;
   L.bytes = 2L * (LROWS * L.qstr + (long)KT * L.qstr + (long)L.RB * 16 * L.ktstr + 2L * LROWS * L.pstr) + 4L * 4 * LROWS;
   return L;
 }
 
-template <int CB>
+template <int CB, int KT>
 __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const u16* __restrict__ qa, const u16* __restrict__ q, long ldq, int H, int dim, int rot, int rank, long Ttot,
     const float* __restrict__ cos_sin, int tab_w, const u16* __restrict__ cache, const int* __restrict__ bt, int bt_w,
     const int* __restrict__ qstart, const int* __restrict__ qlen, const int* __restrict__ ctx,
-    const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, u16* __restrict__ out, int KT,
+    const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, u16* __restrict__ out,
     int tpe, int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int Dpad, int qstr, int ktstr,
     int pstr, int RB) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
@@ -336,8 +336,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     }
     qsh[rr * qstr + c] = f2bf(v);
   }
-  // zero what no staging pass writes: the transposed tile's padded rows and the key rows' padded dims
-  for (int e = tid; e < RB * 16 * ktstr; e += 256) ktr[e] = 0;
+  // zero what no staging pass writes: the key rows' padded dims
   for (int e = tid; e < KT * qstr; e += 256) ksh[e] = 0;
   const int last_row = min(row0 + LROWS, nrows) - 1;
   const int kmax = p0 + tok0 + last_row / H + 1;
@@ -359,24 +358,50 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
   const int ntiles = (kmax + KT - 1) / KT;
   const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * KT;
   const int kend = min(kmax, (int)((long)ntiles * (blockIdx.z + 1) / splits) * KT);
-  const int NKB = KT >> 4;
+  constexpr int NKB = KT >> 4;
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     const int nk = min(KT, kend - k0);
     __syncthreads();
     const int pg0 = k0 >> 4, npg = ((k0 + nk - 1) >> 4) - pg0 + 1;
     const int pg = lane < npg ? btr[pg0 + lane] : 0;
-    for (int kk = wave; kk < KT; kk += 4) {        // a wave per key row; rows past the tile's end are zeros
-      const int kidx = k0 + kk;
+    // a wave per key row, all of a wave's rows in flight at once (the loop is unrolled: KT / 4 rows);
+    // rows past the tile's end are zeros.  Rows of a multiple of 8 entries move 16 bytes per lane.
+    const bool vec8 = (Dp & 7) == 0;
+#pragma unroll
+    for (int r = 0; r < KT / 4; ++r) {
+      const int kk = wave + 4 * r, kidx = k0 + kk;
       const bool live = kk < nk;
       const long page = __shfl(pg, live ? (kidx >> 4) - pg0 : 0);
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(cache + (page * 16 + (kidx & 15)) * Dp);
-      for (int c2 = lane; c2 < (Dp >> 1); c2 += 64) {
-        const uint32_t w = live ? src[c2] : 0u;
-        *reinterpret_cast<uint32_t*>(ksh + kk * qstr + 2 * c2) = w;
-        if (2 * c2 < rank) {
-          ktr[(2 * c2) * ktstr + kk] = (u16)(w & 0xffffu);
-          ktr[(2 * c2 + 1) * ktstr + kk] = (u16)(w >> 16);
+      const u16* srow = cache + (page * 16 + (kidx & 15)) * Dp;
+      if (vec8) {
+        const uint4* src = reinterpret_cast<const uint4*>(srow);
+        for (int c8 = lane; c8 < (Dp >> 3); c8 += 64) {
+          const uint4 w = live ? src[c8] : make_uint4(0u, 0u, 0u, 0u);
+          *reinterpret_cast<uint4*>(ksh + kk * qstr + 8 * c8) = w;
         }
+      } else {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(srow);
+        for (int c2 = lane; c2 < (Dp >> 1); c2 += 64) {
+          const uint32_t w = live ? src[c2] : 0u;
+          *reinterpret_cast<uint32_t*>(ksh + kk * qstr + 2 * c2) = w;
+        }
+      }
+    }
+    __syncthreads();
+    // the latent part once more, transposed ([dim][key]): threads along the dims read 8 keys' entries
+    // (2-byte reads of consecutive halfwords) and write them as one 16-byte vector
+    {
+      const int ndim = RB * 16;
+      for (int e = tid; e < ndim * (KT / 8); e += 256) {
+        const int kg = e / ndim, c = e - kg * ndim;
+        uint32_t w4[4] = {0u, 0u, 0u, 0u};
+        if (c < rank) {
+          const u16* col = ksh + (8 * kg) * qstr + c;
+#pragma unroll
+          for (int x = 0; x < 4; ++x)
+            w4[x] = (uint32_t)col[(2 * x) * qstr] | ((uint32_t)col[(2 * x + 1) * qstr] << 16);
+        }
+        *reinterpret_cast<uint4*>(ktr + c * ktstr + 8 * kg) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
       }
     }
     __syncthreads();
@@ -434,9 +459,7 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
         for (int ks = 0; ks < KT; ks += 32) {
           const bf16x8 ah = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(phi + lr * pstr + ks + 8 * g));
           const bf16x8 al = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(plo + lr * pstr + ks + 8 * g));
-          const uint32_t* b32 = reinterpret_cast<const uint32_t*>(bp + ks);
-          const uint4 bw = make_uint4(b32[0], b32[1], b32[2], b32[3]);
-          const bf16x8 b = __builtin_bit_cast(bf16x8, bw);
+          const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + ks));
           acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, b, acc[j], 0, 0, 0);
           acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, b, acc[j], 0, 0, 0);
         }
@@ -572,20 +595,25 @@ int launch_latent_mfma(dim3 g, hipStream_t st, const u16* qa, const u16* q, long
                        float scale, u16* out, int KT, int tpe, int splits, float* part_o, float* part_ml) {
   const MfmaLds L = mfma_lds(rank, rot, KT);
   const int cbs = (L.RB + 3) / 4;
-#define LATM(CB)                                                                                                       \
+#define LATM2(CB, KTC)                                                                                                 \
   do {                                                                                                                 \
     static long have_ = 48 * 1024;                                                                                     \
     if (L.bytes > have_) {                                                                                             \
-      hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<CB>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
-                          (int)L.bytes);                                                                               \
+      hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<CB, KTC>,                                          \
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.bytes);                                   \
       have_ = L.bytes;                                                                                                 \
     }                                                                                                                  \
-    hipLaunchKernelGGL((latent_attention_mfma_kernel<CB>), g, dim3(256), L.bytes, st, qa, q, ldq, H, dim, rot, rank,   \
-                       Ttot, cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, KT,  \
+    hipLaunchKernelGGL((latent_attention_mfma_kernel<CB, KTC>), g, dim3(256), L.bytes, st, qa, q, ldq, H, dim, rot,    \
+                       rank, Ttot, cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, \
                        tpe, splits, part_o, part_ml, L.Dpad, L.qstr, L.ktstr, L.pstr, L.RB);                           \
+  } while (0)
+#define LATM(CB)                                                                                                       \
+  do {                                                                                                                 \
+    if (KT == 64) LATM2(CB, 64); else LATM2(CB, 32);                                                                   \
   } while (0)
   if (cbs <= 1) LATM(1); else if (cbs <= 2) LATM(2); else if (cbs <= 4) LATM(4); else LATM(8);
 #undef LATM
+#undef LATM2
   if (splits > 1) {
     const long n_rows = (long)g.y * g.x * LROWS;
     hipLaunchKernelGGL(latent_combine_kernel<u16>, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, part_o, part_ml,
