@@ -288,6 +288,28 @@ static inline MfmaLds mfma_lds(int rank, int rot, int KT) {
   return L;
 }
 
+// A key tile's rows into registers: wave w takes rows w, w + 4, ..., a lane 16 bytes of a row (two per
+// row cover up to 1024 entries); rows past `kend` and lanes past the row's end get zeros.
+template <int KT>
+__device__ __forceinline__ void fetch_tile(uint4 (&pf)[KT / 4][2], const u16* __restrict__ cache,
+                                           const int* __restrict__ btr, int k0, int kend, int Dp, int lane, int wave) {
+  const int nk = min(KT, kend - k0);
+  const int pg0 = k0 >> 4, npg = ((k0 + nk - 1) >> 4) - pg0 + 1;
+  const int pg = lane < npg ? btr[pg0 + lane] : 0;
+#pragma unroll
+  for (int r = 0; r < KT / 4; ++r) {
+    const int kk = wave + 4 * r, kidx = k0 + kk;
+    const bool live = kk < nk;
+    const long page = __shfl(pg, live ? (kidx >> 4) - pg0 : 0);
+    const uint4* src = reinterpret_cast<const uint4*>(cache + (page * 16 + (kidx & 15)) * Dp);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c8 = lane + 64 * j;
+      pf[r][j] = (live && c8 < (Dp >> 3)) ? src[c8] : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+}
+
 template <int CB, int KT>
 __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const u16* __restrict__ qa, const u16* __restrict__ q, long ldq, int H, int dim, int rot, int rank, long Ttot,
@@ -359,28 +381,35 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
   const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * KT;
   const int kend = min(kmax, (int)((long)ntiles * (blockIdx.z + 1) / splits) * KT);
   constexpr int NKB = KT >> 4;
+  // rows of a multiple of 8 entries (and at most 1024) move as 16-byte vectors, one tile ahead
+  const bool pre = (Dp & 7) == 0 && Dp <= 1024;
+  uint4 pf[KT / 4][2];
+  if (pre && kbeg < kend) fetch_tile<KT>(pf, cache, btr, kbeg, kend, Dp, lane, wave);
   for (int k0 = kbeg; k0 < kend; k0 += KT) {
     const int nk = min(KT, kend - k0);
     __syncthreads();
-    const int pg0 = k0 >> 4, npg = ((k0 + nk - 1) >> 4) - pg0 + 1;
-    const int pg = lane < npg ? btr[pg0 + lane] : 0;
-    // a wave per key row, all of a wave's rows in flight at once (the loop is unrolled: KT / 4 rows);
-    // rows past the tile's end are zeros.  Rows of a multiple of 8 entries move 16 bytes per lane.
-    const bool vec8 = (Dp & 7) == 0;
+    if (pre) {
+      // this tile's rows were fetched into registers while the previous tile was computed; put them
+      // in LDS and start the next tile's fetch, which the products below then hide
 #pragma unroll
-    for (int r = 0; r < KT / 4; ++r) {
-      const int kk = wave + 4 * r, kidx = k0 + kk;
-      const bool live = kk < nk;
-      const long page = __shfl(pg, live ? (kidx >> 4) - pg0 : 0);
-      const u16* srow = cache + (page * 16 + (kidx & 15)) * Dp;
-      if (vec8) {
-        const uint4* src = reinterpret_cast<const uint4*>(srow);
-        for (int c8 = lane; c8 < (Dp >> 3); c8 += 64) {
-          const uint4 w = live ? src[c8] : make_uint4(0u, 0u, 0u, 0u);
-          *reinterpret_cast<uint4*>(ksh + kk * qstr + 8 * c8) = w;
+      for (int r = 0; r < KT / 4; ++r) {
+        const int kk = wave + 4 * r;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int c8 = lane + 64 * j;
+          if (c8 < (Dp >> 3)) *reinterpret_cast<uint4*>(ksh + kk * qstr + 8 * c8) = pf[r][j];
         }
-      } else {
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(srow);
+      }
+      if (k0 + KT < kend) fetch_tile<KT>(pf, cache, btr, k0 + KT, kend, Dp, lane, wave);
+    } else {
+      const int pg0 = k0 >> 4, npg = ((k0 + nk - 1) >> 4) - pg0 + 1;
+      const int pg = lane < npg ? btr[pg0 + lane] : 0;
+#pragma unroll
+      for (int r = 0; r < KT / 4; ++r) {        // a wave per key row; rows past the tile's end are zeros
+        const int kk = wave + 4 * r, kidx = k0 + kk;
+        const bool live = kk < nk;
+        const long page = __shfl(pg, live ? (kidx >> 4) - pg0 : 0);
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(cache + (page * 16 + (kidx & 15)) * Dp);
         for (int c2 = lane; c2 < (Dp >> 1); c2 += 64) {
           const uint32_t w = live ? src[c2] : 0u;
           *reinterpret_cast<uint32_t*>(ksh + kk * qstr + 2 * c2) = w;
