@@ -67,7 +67,8 @@ int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, 
                          void*, int, hipStream_t);
 int dllm_latent_attention(const void*, const void*, long, int, int, int, int, int, long, const float*, int, const void*,
                           const int*, int, const int*, const int*, const int*, const int*, const int*, int, float, void*,
-                          int, float*, float*, int, hipStream_t);
+                          int, float*, float*, int, int, hipStream_t);
+int dllm_latent_mfma_ok(int, int, int);
 int dllm_car_alloc(long, void**);
 int dllm_car_get_handle(void*, char*);
 int dllm_car_handle_size();
@@ -1484,8 +1485,11 @@ void latent_kv_write(torch::Tensor ckv, int64_t rank, torch::Tensor w, double ep
 void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t rot, torch::Tensor pos, torch::Tensor cos_sin,
                       torch::Tensor cache, torch::Tensor bt, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
                       torch::Tensor tile_seq, torch::Tensor tile_tok0, double scale, torch::Tensor out, int64_t splits,
-                      c10::optional<torch::Tensor> part_o, c10::optional<torch::Tensor> part_ml, bool mfma) {
+                      c10::optional<torch::Tensor> part_o, c10::optional<torch::Tensor> part_ml, bool mfma,
+                      int64_t rows) {
   const bool f = act_f32(qa, "qa");
+  TORCH_CHECK(rows == 16 || (rows == 32 && mfma && !f && dllm_latent_mfma_ok((int)qa.size(2), (int)rot, 32)),
+              "rows per workgroup: 16, or 32 where the matrix-core kernel takes the shape");
   TORCH_CHECK(qa.dim() == 3 && qa.is_contiguous(), "qa [H, T, rank] contiguous");
   const int64_t H = qa.size(0), T = qa.size(1), rank = qa.size(2);
   TORCH_CHECK(q.is_cuda() && q.scalar_type() == qa.scalar_type(), "q dtype");
@@ -1510,8 +1514,8 @@ void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t ro
     TORCH_CHECK(part_o && part_ml, "split partial buffers");
     check_f32(*part_o, "part_o");
     check_f32(*part_ml, "part_ml");
-    const int64_t gx = ((H >= 16 ? 1 : 16 / H) * H + 15) / 16, rows = tile_seq.numel() * gx * 16 * splits;
-    TORCH_CHECK(part_o->numel() >= rows * rank && part_ml->numel() >= rows * 2, "split partial buffers too small");
+    const int64_t gx = ((H >= rows ? 1 : rows / H) * H + rows - 1) / rows, prow = tile_seq.numel() * gx * rows * splits;
+    TORCH_CHECK(part_o->numel() >= prow * rank && part_ml->numel() >= prow * 2, "split partial buffers too small");
     po = part_o->data_ptr<float>();
     pml = part_ml->data_ptr<float>();
   }
@@ -1519,7 +1523,7 @@ void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t ro
                            cos_sin.data_ptr<float>(), (int)cos_sin.size(1), cache.data_ptr(), bt.data_ptr<int>(),
                            (int)bt.size(1), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                            tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), (float)scale,
-                           out.data_ptr(), (int)splits, po, pml, mfma ? 1 : 0, stream()),
+                           out.data_ptr(), (int)splits, po, pml, mfma ? 1 : 0, (int)rows, stream()),
      "latent_attention");
 }
 }  // namespace
@@ -1538,7 +1542,9 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("latent_attention", &latent_attention, py::arg("qa"), py::arg("q"), py::arg("dim"), py::arg("rot"),
         py::arg("positions"), py::arg("cos_sin"), py::arg("cache"), py::arg("block_tables"), py::arg("qstart"),
         py::arg("qlen"), py::arg("ctx"), py::arg("tile_seq"), py::arg("tile_tok0"), py::arg("scale"), py::arg("out"),
-        py::arg("splits") = 1, py::arg("part_o") = py::none(), py::arg("part_ml") = py::none(), py::arg("mfma") = true);
+        py::arg("splits") = 1, py::arg("part_o") = py::none(), py::arg("part_ml") = py::none(), py::arg("mfma") = true,
+        py::arg("rows") = 16);
+  m.def("latent_mfma_ok", [](int64_t rank, int64_t rot, int64_t rows) { return dllm_latent_mfma_ok((int)rank, (int)rot, (int)rows) != 0; });
   m.def("encoder_attention", &encoder_attention);
   m.def("embed_ln", &embed_ln);
   m.def("moe_ffn", &moe_ffn, py::arg("x"), py::arg("ids"), py::arg("wts"), py::arg("w13"), py::arg("w2"), py::arg("out"),

@@ -277,14 +277,14 @@ __device__ __forceinline__ float row16_add(float v) {
 }
 
 struct MfmaLds { int Dpad, qstr, ktstr, pstr, RB; long bytes; };
-static inline MfmaLds mfma_lds(int rank, int rot, int KT) {
+static inline MfmaLds mfma_lds(int rank, int rot, int KT, int rows = LROWS) {
   MfmaLds L;
   L.Dpad = (rank + rot + 31) & ~31;
   L.qstr = L.Dpad + 8;
   L.ktstr = KT + 8;
   L.pstr = KT + 8;
   L.RB = (rank + 15) / 16;
-  L.bytes = 2L * (LROWS * L.qstr + (long)KT * L.qstr + (long)L.RB * 16 * L.ktstr + 2L * LROWS * L.pstr) + 4L * 4 * LROWS;
+  L.bytes = 2L * (rows * L.qstr + (long)KT * L.qstr + (long)L.RB * 16 * L.ktstr + 2L * rows * L.pstr) + 4L * 4 * rows;
   return L;
 }
 
@@ -310,7 +310,10 @@ __device__ __forceinline__ void fetch_tile(uint4 (&pf)[KT / 4][2], const u16* __
   }
 }
 
-template <int CB, int KT>
+// LR: 16-row blocks per workgroup (1: decode steps and short portions; 2: prompt portions, where the
+// tile's staging, transposition and barriers then serve 32 rows and every wave has a score task at
+// 32-key tiles).  Score tasks (row block, 16 keys) are dealt to the waves round-robin.
+template <int CB, int KT, int LR>
 __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const u16* __restrict__ qa, const u16* __restrict__ q, long ldq, int H, int dim, int rot, int rank, long Ttot,
     const float* __restrict__ cos_sin, int tab_w, const u16* __restrict__ cache, const int* __restrict__ bt, int bt_w,
@@ -318,6 +321,9 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
     const int* __restrict__ tile_seq, const int* __restrict__ tile_tok0, float scale, u16* __restrict__ out,
     int tpe, int splits, float* __restrict__ part_o, float* __restrict__ part_ml, int Dpad, int qstr, int ktstr,
     int pstr, int RB) {
+  constexpr int RPB = 16 * LR;                      // rows per workgroup
+  constexpr int NKB = KT >> 4;                      // 16-key blocks per tile
+  constexpr int NT = (LR * NKB + 3) / 4;            // score tasks per wave
   extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
   const int entry = blockIdx.y;
   const int s = tile_seq[entry];
@@ -327,20 +333,20 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
   if (tok0 >= n) return;
   const int ntok = min(tpe, n - tok0);
   const int nrows = ntok * H;
-  const int row0 = blockIdx.x * LROWS;
+  const int row0 = blockIdx.x * RPB;
   if (row0 >= nrows) return;
   const int q0 = qstart[s], p0 = ctx[s] - n;
   const int Dp = rank + rot;
-  u16* qsh = reinterpret_cast<u16*>(smraw);             // [16][qstr]
-  u16* ksh = qsh + LROWS * qstr;                        // [KT][qstr]
+  u16* qsh = reinterpret_cast<u16*>(smraw);             // [RPB][qstr]
+  u16* ksh = qsh + RPB * qstr;                          // [KT][qstr]
   u16* ktr = ksh + KT * qstr;                           // [RB * 16][ktstr]: latent part transposed
-  u16* phi = ktr + RB * 16 * ktstr;                     // [16][pstr]
-  u16* plo = phi + LROWS * pstr;
-  float* wred = reinterpret_cast<float*>(plo + LROWS * pstr);   // [4][16]
+  u16* phi = ktr + RB * 16 * ktstr;                     // [RPB][pstr]
+  u16* plo = phi + RPB * pstr;
+  float* wred = reinterpret_cast<float*>(plo + RPB * pstr);   // [4][RPB]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 15, g = lane >> 4;
   const int half = rot >> 1;
-  for (int e = tid; e < LROWS * Dpad; e += 256) {
+  for (int e = tid; e < RPB * Dpad; e += 256) {
     const int rr = e / Dpad, c = e - rr * Dpad, row = row0 + rr;
     float v = 0.f;
     if (row < nrows && c < Dp) {
@@ -360,27 +366,29 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
   }
   // zero what no staging pass writes: the key rows' padded dims
   for (int e = tid; e < KT * qstr; e += 256) ksh[e] = 0;
-  const int last_row = min(row0 + LROWS, nrows) - 1;
+  const int last_row = min(row0 + RPB, nrows) - 1;
   const int kmax = p0 + tok0 + last_row / H + 1;
-  int rpos[4];
-  bool rok[4];
+  int rpos[LR][4];
+  bool rok[LR][4];
+  float m[LR][4], l[LR][4];
+  f32x4 acc[CB][LR];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = row0 + 4 * g + i;
-    rok[i] = row < nrows;
-    rpos[i] = p0 + tok0 + (rok[i] ? row / H : 0);
+  for (int b = 0; b < LR; ++b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = row0 + 16 * b + 4 * g + i;
+      rok[b][i] = row < nrows;
+      rpos[b][i] = p0 + tok0 + (rok[b][i] ? row / H : 0);
+      m[b][i] = -INFINITY;
+      l[b][i] = 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < CB; ++j) acc[j][b] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  float m[4], l[4];
-  f32x4 acc[CB];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) { m[i] = -INFINITY; l[i] = 0.f; }
-#pragma unroll
-  for (int j = 0; j < CB; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int* btr = bt + (long)s * bt_w;
   const int ntiles = (kmax + KT - 1) / KT;
   const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * KT;
   const int kend = min(kmax, (int)((long)ntiles * (blockIdx.z + 1) / splits) * KT);
-  constexpr int NKB = KT >> 4;
   // rows of a multiple of 8 entries (and at most 1024) move as 16-byte vectors, one tile ahead
   const bool pre = (Dp & 7) == 0 && Dp <= 1024;
   uint4 pf[KT / 4][2];
@@ -434,46 +442,80 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
       }
     }
     __syncthreads();
-    // scores of this wave's 16 keys
-    f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
-    if (wave < NKB) {
-      const u16* ap = qsh + lr * qstr + 8 * g;
-      const u16* bp = ksh + (16 * wave + lr) * qstr + 8 * g;
-      for (int st = 0; st < Dpad; st += 32) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ap + st));
-        const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + st));
-        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, sacc, 0, 0, 0);
+    // scores: task t of this wave is (row block, key block) number wave + 4 t
+    float sv[NT][4];
+    bool vis[NT][4];
+    float wm[LR][4];
+#pragma unroll
+    for (int b = 0; b < LR; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) wm[b][i] = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int task = wave + 4 * t;
+      const bool on = task < LR * NKB;
+      const int rb = on ? task / NKB : 0, kb = on ? task % NKB : 0;
+      f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+      if (on) {
+        const u16* ap = qsh + (16 * rb + lr) * qstr + 8 * g;
+        const u16* bp = ksh + (16 * kb + lr) * qstr + 8 * g;
+        for (int st = 0; st < Dpad; st += 32) {
+          const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ap + st));
+          const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + st));
+          sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, sacc, 0, 0, 0);
+        }
+      }
+      const int kidx = k0 + 16 * kb + lr;
+#pragma unroll
+      for (int b = 0; b < LR; ++b) {          // (static indexing of the per-row-block registers)
+        if (b == rb) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            vis[t][i] = on && kidx < kend && rok[b][i] && kidx <= rpos[b][i];
+            sv[t][i] = vis[t][i] ? sacc[i] * scale : -INFINITY;
+            wm[b][i] = fmaxf(wm[b][i], row16_max(sv[t][i]));
+          }
+        }
       }
     }
-    const int kidx = k0 + 16 * wave + lr;
-    float sv[4];
-    bool vis[4];
+    if (lr == 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      vis[i] = wave < NKB && kidx < kend && rok[i] && kidx <= rpos[i];
-      sv[i] = vis[i] ? sacc[i] * scale : -INFINITY;
-      const float wm = row16_max(sv[i]);
-      if (lr == 0) wred[wave * LROWS + 4 * g + i] = wm;
+      for (int b = 0; b < LR; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wred[wave * RPB + 16 * b + 4 * g + i] = wm[b][i];
     }
     __syncthreads();
-    float alpha[4];
+    float alpha[LR][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = 4 * g + i;
-      const float tm = fmaxf(fmaxf(wred[r], wred[LROWS + r]), fmaxf(wred[2 * LROWS + r], wred[3 * LROWS + r]));
-      const float mn = fmaxf(m[i], tm);
-      float p = 0.f;
-      alpha[i] = 1.f;
-      if (mn != -INFINITY) {
-        p = vis[i] ? expf(sv[i] - mn) : 0.f;
-        alpha[i] = expf(m[i] - mn);
-        m[i] = mn;
+    for (int b = 0; b < LR; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = 16 * b + 4 * g + i;
+        const float tm = fmaxf(fmaxf(wred[r], wred[RPB + r]), fmaxf(wred[2 * RPB + r], wred[3 * RPB + r]));
+        const float mn = fmaxf(m[b][i], tm);
+        alpha[b][i] = mn != -INFINITY ? expf(m[b][i] - mn) : 1.f;
+        m[b][i] = mn;
+        l[b][i] *= alpha[b][i];
       }
-      l[i] = l[i] * alpha[i] + p;
-      if (wave < NKB) {
-        const u16 hi = f2bf(p);
-        phi[r * pstr + 16 * wave + lr] = hi;
-        plo[r * pstr + 16 * wave + lr] = f2bf(p - bf2f(hi));
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int task = wave + 4 * t;
+      if (task < LR * NKB) {
+        const int rb = task / NKB, kb = task % NKB;
+#pragma unroll
+        for (int b = 0; b < LR; ++b) {
+          if (b == rb) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float p = (vis[t][i] && m[b][i] != -INFINITY) ? expf(sv[t][i] - m[b][i]) : 0.f;
+              l[b][i] += p;
+              const u16 hi = f2bf(p);
+              const int r = 16 * b + 4 * g + i;
+              phi[r * pstr + 16 * kb + lr] = hi;
+              plo[r * pstr + 16 * kb + lr] = f2bf(p - bf2f(hi));
+            }
+          }
+        }
       }
     }
     __syncthreads();
@@ -483,14 +525,20 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
       const int cb = wave + 4 * j;
       if (cb < RB) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[j][i] *= alpha[i];
+        for (int b = 0; b < LR; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[j][b][i] *= alpha[b][i];
         const u16* bp = ktr + (cb * 16 + lr) * ktstr + 8 * g;
         for (int ks = 0; ks < KT; ks += 32) {
-          const bf16x8 ah = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(phi + lr * pstr + ks + 8 * g));
-          const bf16x8 al = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(plo + lr * pstr + ks + 8 * g));
-          const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + ks));
-          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, b, acc[j], 0, 0, 0);
-          acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, b, acc[j], 0, 0, 0);
+          const bf16x8 bv = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + ks));
+#pragma unroll
+          for (int b = 0; b < LR; ++b) {
+            const int ro = (16 * b + lr) * pstr + ks + 8 * g;
+            const bf16x8 ah = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(phi + ro));
+            const bf16x8 al = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(plo + ro));
+            acc[j][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bv, acc[j][b], 0, 0, 0);
+            acc[j][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, bv, acc[j][b], 0, 0, 0);
+          }
         }
       }
     }
@@ -498,41 +546,40 @@ __global__ void __launch_bounds__(256) latent_attention_mfma_kernel(
   // row sums: over the 16 lanes of a row group, then over the waves
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float t = row16_add(l[i]);
-    if (lr == 0) wred[wave * LROWS + 4 * g + i] = t;
-  }
-  __syncthreads();
-  float lt[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = 4 * g + i;
-    lt[i] = wred[r] + wred[LROWS + r] + wred[2 * LROWS + r] + wred[3 * LROWS + r];
-  }
-  if (splits > 1) {
+  for (int b = 0; b < LR; ++b)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const long pr = (((long)entry * gridDim.x + blockIdx.x) * LROWS + 4 * g + i) * splits + blockIdx.z;
-      if (wave == 0 && lr == 0) { part_ml[2 * pr] = m[i]; part_ml[2 * pr + 1] = lt[i]; }
-#pragma unroll
-      for (int j = 0; j < CB; ++j) {
-        const int c = (wave + 4 * j) * 16 + lr;
-        if (wave + 4 * j < RB && c < rank) part_o[pr * rank + c] = acc[j][i];
-      }
+      const float t = row16_add(l[b][i]);
+      if (lr == 0) wred[wave * RPB + 16 * b + 4 * g + i] = t;
     }
-    return;
-  }
+  __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = row0 + 4 * g + i;
-    if (row >= nrows) continue;
-    const long tok = q0 + tok0 + row / H;
-    const int h = row % H;
-    const float inv = lt[i] > 0.f ? 1.f / lt[i] : 0.f;
+  for (int b = 0; b < LR; ++b) {
 #pragma unroll
-    for (int j = 0; j < CB; ++j) {
-      const int c = (wave + 4 * j) * 16 + lr;
-      if (wave + 4 * j < RB && c < rank) out[((long)h * Ttot + tok) * rank + c] = f2bf(acc[j][i] * inv);
+    for (int i = 0; i < 4; ++i) {
+      const int r = 16 * b + 4 * g + i;
+      const float lt = wred[r] + wred[RPB + r] + wred[2 * RPB + r] + wred[3 * RPB + r];
+      if (splits > 1) {
+        const long pr = (((long)entry * gridDim.x + blockIdx.x) * RPB + r) * splits + blockIdx.z;
+        if (wave == 0 && lr == 0) { part_ml[2 * pr] = m[b][i]; part_ml[2 * pr + 1] = lt; }
+#pragma unroll
+        for (int j = 0; j < CB; ++j) {
+          const int c = (wave + 4 * j) * 16 + lr;
+          if (wave + 4 * j < RB && c < rank) part_o[pr * rank + c] = acc[j][b][i];
+        }
+      } else {
+        const int row = row0 + r;
+        if (row < nrows) {
+          const long tok = q0 + tok0 + row / H;
+          const int h = row % H;
+          const float inv = lt > 0.f ? 1.f / lt : 0.f;
+#pragma unroll
+          for (int j = 0; j < CB; ++j) {
+            const int c = (wave + 4 * j) * 16 + lr;
+            if (wave + 4 * j < RB && c < rank) out[((long)h * Ttot + tok) * rank + c] = f2bf(acc[j][b][i] * inv);
+          }
+        }
+      }
     }
   }
 }
@@ -544,17 +591,17 @@ __global__ void __launch_bounds__(256) latent_combine_kernel(const float* __rest
                                                              int H, int rank, long Ttot, const int* __restrict__ qstart,
                                                              const int* __restrict__ qlen, const int* __restrict__ tile_seq,
                                                              const int* __restrict__ tile_tok0, int tpe, long n_rows,
-                                                             T* __restrict__ out) {
+                                                             T* __restrict__ out, int rpb) {
   const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;
   const int lane = threadIdx.x & 63;
-  const int rl = (int)(r % LROWS);
-  const long eb = r / LROWS;
+  const int rl = (int)(r % rpb);
+  const long eb = r / rpb;
   const int bx = (int)(eb % gx), entry = (int)(eb / gx);
   const int s = tile_seq[entry];
   const int n = qlen[s], tok0 = tile_tok0[entry];
   if (n <= 0 || tok0 >= n) return;
-  const int row = bx * LROWS + rl;
+  const int row = bx * rpb + rl;
   if (row >= min(tpe, n - tok0) * H) return;
   const float* ml = part_ml + 2 * r * splits;
   float M = -INFINITY;
@@ -611,7 +658,7 @@ int launch_latent(int ri, dim3 g, long lds, hipStream_t st, const T* qa, const T
   if (splits > 1) {
     const long n_rows = (long)g.y * g.x * LROWS;
     hipLaunchKernelGGL(latent_combine_kernel<T>, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, part_o, part_ml, splits,
-                       (int)g.x, H, rank, Ttot, qstart, qlen, tile_seq, tile_tok0, tpe, n_rows, out);
+                       (int)g.x, H, rank, Ttot, qstart, qlen, tile_seq, tile_tok0, tpe, n_rows, out, LROWS);
   }
   return (int)hipGetLastError();
 }
@@ -621,20 +668,24 @@ namespace {
 int launch_latent_mfma(dim3 g, hipStream_t st, const u16* qa, const u16* q, long ldq, int H, int dim, int rot, int rank,
                        long Ttot, const float* cos_sin, int tab_w, const u16* cache, const int* bt, int bt_w,
                        const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
-                       float scale, u16* out, int KT, int tpe, int splits, float* part_o, float* part_ml) {
-  const MfmaLds L = mfma_lds(rank, rot, KT);
+                       float scale, u16* out, int KT, int tpe, int splits, float* part_o, float* part_ml, int rows) {
+  const MfmaLds L = mfma_lds(rank, rot, KT, rows);
   const int cbs = (L.RB + 3) / 4;
-#define LATM2(CB, KTC)                                                                                                 \
+#define LATM3(CB, KTC, LRC)                                                                                                 \
   do {                                                                                                                 \
     static long have_ = 48 * 1024;                                                                                     \
     if (L.bytes > have_) {                                                                                             \
-      hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<CB, KTC>,                                          \
+      hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<CB, KTC, LRC>,                                     \
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.bytes);                                   \
       have_ = L.bytes;                                                                                                 \
     }                                                                                                                  \
-    hipLaunchKernelGGL((latent_attention_mfma_kernel<CB, KTC>), g, dim3(256), L.bytes, st, qa, q, ldq, H, dim, rot,    \
+    hipLaunchKernelGGL((latent_attention_mfma_kernel<CB, KTC, LRC>), g, dim3(256), L.bytes, st, qa, q, ldq, H, dim, rot, \
                        rank, Ttot, cos_sin, tab_w, cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, out, \
                        tpe, splits, part_o, part_ml, L.Dpad, L.qstr, L.ktstr, L.pstr, L.RB);                           \
+  } while (0)
+#define LATM2(CB, KTC)                                                                                                 \
+  do {                                                                                                                 \
+    if (rows == 32) LATM3(CB, KTC, 2); else LATM3(CB, KTC, 1);                                                         \
   } while (0)
 #define LATM(CB)                                                                                                       \
   do {                                                                                                                 \
@@ -643,37 +694,40 @@ int launch_latent_mfma(dim3 g, hipStream_t st, const u16* qa, const u16* q, long
   if (cbs <= 1) LATM(1); else if (cbs <= 2) LATM(2); else if (cbs <= 4) LATM(4); else LATM(8);
 #undef LATM
 #undef LATM2
+#undef LATM3
   if (splits > 1) {
-    const long n_rows = (long)g.y * g.x * LROWS;
+    const long n_rows = (long)g.y * g.x * rows;
     hipLaunchKernelGGL(latent_combine_kernel<u16>, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, part_o, part_ml,
-                       splits, (int)g.x, H, rank, Ttot, qstart, qlen, tile_seq, tile_tok0, tpe, n_rows, out);
+                       splits, (int)g.x, H, rank, Ttot, qstart, qlen, tile_seq, tile_tok0, tpe, n_rows, out, rows);
   }
   return (int)hipGetLastError();
 }
 }  // namespace
 
-// 1 when the matrix-core kernel takes this shape (bf16, even widths, a 32-key tile fits the LDS)
-extern "C" int dllm_latent_mfma_ok(int rank, int rot) {
-  if ((rank & 1) || (rot & 1) || rank < 2 || rank > 512) return 0;
-  return mfma_lds(rank, rot, 32).bytes <= 150 * 1024;
+// 1 when the matrix-core kernel takes this shape with `rows` (16 or 32) rows per workgroup (bf16, even
+// widths, a 32-key tile fits the LDS)
+extern "C" int dllm_latent_mfma_ok(int rank, int rot, int rows) {
+  if ((rank & 1) || (rot & 1) || rank < 2 || rank > 512 || (rows != 16 && rows != 32)) return 0;
+  return mfma_lds(rank, rot, 32, rows).bytes <= 150 * 1024;
 }
 
 extern "C" int dllm_latent_attention(const void* qa, const void* q, long ldq, int f32, int H, int dim, int rot, int rank,
                                      long Ttot, const float* cos_sin, int tab_w, const void* cache, const int* bt,
                                      int bt_w, const int* qstart, const int* qlen, const int* ctx, const int* tile_seq,
                                      const int* tile_tok0, int n_entries, float scale, void* out, int splits,
-                                     float* part_o, float* part_ml, int mfma, hipStream_t st) {
+                                     float* part_o, float* part_ml, int mfma, int rows, hipStream_t st) {
   if (n_entries <= 0 || Ttot <= 0) return 0;
   if (rank < 1 || rank > 512 || rot < 0 || (rot & 1) || rot > tab_w || H < 1) return -1;
   if (splits < 1 || (splits > 1 && (!part_o || !part_ml))) return -3;
-  if (mfma && !f32 && dllm_latent_mfma_ok(rank, rot)) {
-    const int KTm = mfma_lds(rank, rot, 64).bytes <= 150 * 1024 ? 64 : 32;
-    const int tpe_m = H >= 16 ? 1 : 16 / H;
-    const dim3 gm((tpe_m * H + LROWS - 1) / LROWS, n_entries, splits);
+  if (mfma && !f32 && dllm_latent_mfma_ok(rank, rot, rows)) {
+    const int KTm = mfma_lds(rank, rot, 64, rows).bytes <= 150 * 1024 ? 64 : 32;
+    const int tpe_m = H >= rows ? 1 : rows / H;
+    const dim3 gm((tpe_m * H + rows - 1) / rows, n_entries, splits);
     return launch_latent_mfma(gm, st, (const u16*)qa, (const u16*)q, ldq, H, dim, rot, rank, Ttot, cos_sin, tab_w,
                               (const u16*)cache, bt, bt_w, qstart, qlen, ctx, tile_seq, tile_tok0, scale, (u16*)out, KTm,
-                              tpe_m, splits, part_o, part_ml);
+                              tpe_m, splits, part_o, part_ml, rows);
   }
+  if (rows != LROWS) return -4;   // only the matrix-core kernel has the 32-row form
   // key rows in LDS: an odd stride for 4-byte reads; when the row length is a multiple of 4 a stride
   // that is 4 x odd, so a lane's 16-byte reads are aligned and spread over all banks
   const int Dp = rank + rot, vec = (Dp & 3) == 0;

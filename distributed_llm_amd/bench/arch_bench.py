@@ -154,10 +154,11 @@ def kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 2048) -> Di
         from ..models.llama import AttnMeta
         meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=cx, tile_seq=None, tile_tok0=None,
                         last_idx=None, host_qlen=qlens)
-        ts, tt = meta.latent_tiles(Hl, dev)
+        lrows = seqmix.latent_rows(qa, r, dr, n, S)
+        ts, tt = meta.latent_tiles(Hl, dev, lrows)
         keys = sum((a + (m + 1) / 2) * m for a, m in zip(starts, qlens))     # causal (query, key) pairs
         rec(f"latent_attention_{tag}",
-            _timed(lambda: seqmix.latent_attention(qa, q, dl, dr, pos, tab2, cache, bt, qstart, qlen, cx, ts, tt, 0.1), 3),
+            _timed(lambda: seqmix.latent_attention(qa, q, dl, dr, pos, tab2, cache, bt, qstart, qlen, cx, ts, tt, 0.1, rows=lrows), 3),
             (sum(a + m for a, m in zip(starts, qlens)) * (r + dr) * 2 + n * Hl * r * 4),
             keys * Hl * (2 * (r + dr) + 2 * r), PEAK_BF16)
     return res

@@ -263,9 +263,11 @@ class HybridModel:
                                cache[0])
         qn = q.view(T, H, m.dim + m.rot_dim)[:, :, :m.dim].transpose(0, 1)
         qa = torch.bmm(qn, L["uk"])                                     # key up-projection absorbed: [H, T, rank]
-        ts, tr = meta.latent_tiles(H, self.device)
+        rows = (seqmix.LAT_ROWS if meta.host_qlen is None else
+                seqmix.latent_rows(x, m.kv_rank, m.rot_dim, T, len(meta.host_qlen)))
+        ts, tr = meta.latent_tiles(H, self.device, rows)
         lat = seqmix.latent_attention(qa, q, m.dim, m.rot_dim, positions, table, cache[0], meta.block_tables,
-                                      meta.qstart, meta.qlen, meta.ctx, ts, tr, m.scale)
+                                      meta.qstart, meta.qlen, meta.ctx, ts, tr, m.scale, rows=rows)
         o = torch.bmm(lat, L["uvT"])                                    # [H, T, vdim]
         return _mm(o.transpose(0, 1).reshape(T, H * m.vdim), L["o"])
 

@@ -66,15 +66,16 @@ class AttnMeta:
     host_qlen: Optional[List[int]] = None      # prefill: new tokens per sequence, on the host
     _lat: Optional[Dict[int, Tuple[torch.Tensor, torch.Tensor]]] = None
 
-    def latent_tiles(self, heads: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(sequence, first token) entries of the latent attention kernel for ``heads`` heads: an
-        entry covers max(1, 16 // heads) tokens.  Decode steps (one token per sequence) use the
-        step's own tile table; prefill builds one per head count from ``host_qlen``."""
+    def latent_tiles(self, heads: int, device, rows: int = 16) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(sequence, first token) entries of the latent attention kernel for ``heads`` heads and
+        ``rows`` (token, head) rows per workgroup: an entry covers max(1, rows // heads) tokens.
+        Decode steps (one token per sequence) use the step's own tile table; prefill builds one per
+        entry width from ``host_qlen``."""
         if self.host_qlen is None:
             return self.tile_seq, self.tile_tok0
         if self._lat is None:
             self._lat = {}
-        tpe = max(1, 16 // heads)
+        tpe = max(1, rows // heads)
         if tpe not in self._lat:
             ts, tt = [], []
             for i, n in enumerate(self.host_qlen):

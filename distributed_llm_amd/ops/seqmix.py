@@ -107,15 +107,28 @@ LAT_SPLIT_TARGET = 512     # workgroups a small latent-attention grid is split u
 LAT_SPLIT_MAX = 16
 
 
-def latent_splits(n_entries: int, heads: int) -> int:
+def latent_splits(n_entries: int, heads: int, rows: int = LAT_ROWS) -> int:
     """Key splits of a latent attention launch: grids with fewer than ``LAT_SPLIT_TARGET`` workgroups
     (decode steps, short portions) split every row's keys over up to ``LAT_SPLIT_MAX`` workgroups."""
-    gx = ((1 if heads >= 16 else 16 // heads) * heads + LAT_ROWS - 1) // LAT_ROWS
+    gx = ((1 if heads >= rows else rows // heads) * heads + rows - 1) // rows
     return max(1, min(LAT_SPLIT_MAX, LAT_SPLIT_TARGET // max(1, n_entries * gx)))
 
 
+def latent_rows(x: torch.Tensor, rank: int, rot_dim: int, tokens: int, seqs: int) -> int:
+    """(token, head) rows per workgroup of a latent attention launch: 32 for prompt portions of bf16
+    models on the GPU where the matrix-core kernel's 32-row form fits the LDS, else 16.  The step's
+    tile table (AttnMeta.latent_tiles) must be built for the same number."""
+    if not x.is_cuda or x.dtype != torch.bfloat16 or tokens < 8 * max(1, seqs):
+        return LAT_ROWS
+    if os.environ.get("DLLM_LATENT_MFMA", "1") != "1" or os.environ.get("DLLM_LATENT_ROWS", "32") != "32":
+        return LAT_ROWS
+    ext = _native(x)
+    return 32 if ext is not None and ext.latent_mfma_ok(int(rank), int(rot_dim), 32) else LAT_ROWS
+
+
 def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_tables, qstart, qlen, ctx, tile_seq,
-                     tile_tok0, scale, splits: Optional[int] = None, mfma: Optional[bool] = None) -> torch.Tensor:
+                     tile_tok0, scale, splits: Optional[int] = None, mfma: Optional[bool] = None,
+                     rows: int = LAT_ROWS) -> torch.Tensor:
     """``mfma`` (GPU, bf16): the matrix-core kernel (default where the shape fits it;
     ``DLLM_LATENT_MFMA=0`` or ``mfma=False`` keeps the vector-ALU kernel that f32 models run)."""
     ext = _native(qa)
@@ -124,17 +137,17 @@ def latent_attention(qa, q, dim, rot_dim, positions, cos_sin, cache, block_table
                                     scale)
     out = torch.zeros_like(qa)
     H, n_entries = qa.shape[0], int(tile_seq.numel())
-    sp = latent_splits(n_entries, H) if splits is None else int(splits)
+    sp = latent_splits(n_entries, H, rows) if splits is None else int(splits)
     po = pml = None
     if sp > 1:
-        gx = ((1 if H >= 16 else 16 // H) * H + LAT_ROWS - 1) // LAT_ROWS
-        rows = n_entries * gx * LAT_ROWS * sp
-        po = torch.empty(rows * qa.shape[2], dtype=torch.float32, device=qa.device)
-        pml = torch.empty(rows * 2, dtype=torch.float32, device=qa.device)
+        gx = ((1 if H >= rows else rows // H) * H + rows - 1) // rows
+        prow = n_entries * gx * rows * sp
+        po = torch.empty(prow * qa.shape[2], dtype=torch.float32, device=qa.device)
+        pml = torch.empty(prow * 2, dtype=torch.float32, device=qa.device)
     if mfma is None:
         mfma = os.environ.get("DLLM_LATENT_MFMA", "1") == "1"
     ext.latent_attention(qa, q, int(dim), int(rot_dim), positions, cos_sin, cache, block_tables, qstart, qlen, ctx,
-                         tile_seq, tile_tok0, float(scale), out, sp, po, pml, bool(mfma))
+                         tile_seq, tile_tok0, float(scale), out, sp, po, pml, bool(mfma), int(rows))
     return out
 
 

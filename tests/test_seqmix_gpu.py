@@ -113,11 +113,12 @@ def test_retention(dt, case, H, d, dv, rot, chunked):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES)
 @pytest.mark.parametrize("splits", [1, 3, 16])
-@pytest.mark.parametrize("mfma", [False, True])
+@pytest.mark.parametrize("mfma", [False, True, 32])
 @pytest.mark.parametrize("H,dim,rot,rank", [(8, 32, 16, 96), (3, 16, 8, 40), (20, 32, 16, 128), (1, 8, 64, 512), (2, 8, 6, 70)])
 def test_latent_attention(dt, case, H, dim, rot, rank, splits, mfma):
     if mfma and dt != torch.bfloat16:
         pytest.skip("the matrix-core kernel serves bf16 models")
+    wg_rows = 32 if mfma == 32 else 16
     torch.manual_seed(3)
     qlens, starts = case
     T, qstart, qlen, ctx, rows, pos = batch(qlens, starts)
@@ -146,8 +147,8 @@ def test_latent_attention(dt, case, H, dim, rot, rank, splits, mfma):
     from distributed_llm_amd.models.llama import AttnMeta
     meta = AttnMeta(slots=None, block_tables=perm, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
                     last_idx=None, host_qlen=qlens)
-    ts, tt = meta.latent_tiles(H, DEV)
-    o1 = seqmix.latent_attention(qa, q, dim, rot, pos, table, cache2, perm, qstart, qlen, ctx, ts, tt, 0.2, splits=splits, mfma=mfma)
+    ts, tt = meta.latent_tiles(H, DEV, wg_rows)
+    o1 = seqmix.latent_attention(qa, q, dim, rot, pos, table, cache2, perm, qstart, qlen, ctx, ts, tt, 0.2, splits=splits, mfma=bool(mfma), rows=wg_rows)
     o2 = ref.latent_attention(qa, q, dim, rot, pos, table, cache2, perm, qstart, qlen, ctx, 0.2)
     torch.testing.assert_close(o1.float(), o2.float(), **tol(dt))
 
