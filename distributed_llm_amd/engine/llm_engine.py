@@ -1771,6 +1771,12 @@ class LLMEngine:
     def _feed(self, entries, end) -> torch.Tensor:
         seqs: List[_Seq] = []
         now = time.perf_counter()
+        if not entries:                 # a step that only ends requests
+            for key in end:
+                s = self._streams.pop(key, None)
+                if s is not None:
+                    self._release(s)
+            return torch.empty((0, self.cfg.vocab))
         for key, toks, _ in entries:
             toks = [int(t) for t in toks]
             if not toks:
