@@ -57,10 +57,26 @@ int dllm_selective_scan(const void*, const void*, int, const float*, const float
                         int, int, hipStream_t);
 long dllm_retention_lds(int, int);
 int dllm_retention(const void*, long, int, int, int, int, const float*, int, int, const float*, float*, float,
-                   const int*, const int*, const int*, const int*, void*, int, hipStream_t);
+                   const int*, const int*, const int*, const int*, void*, int, int, float, float*, hipStream_t);
 long dllm_retention_chunk_lds(int);
 int dllm_retention_chunked(const void*, long, int, int, int, int, const float*, int, int, const float*, float*, float,
-                           const int*, const int*, const int*, const int*, float*, void*, int, long, hipStream_t);
+                           const int*, const int*, const int*, const int*, float*, void*, int, long, int, float, int,
+                           hipStream_t);
+int dllm_heads_norm_gate(const float*, const void*, long, int, long, int, const float*, float, const int*, const int*, int,
+                         void*, long, hipStream_t);
+int dllm_resadd_norm(const void*, long, const void*, long, int, const float*, const float*, const float*, float*,
+                     const float*, void*, int, int, float, hipStream_t);
+int dllm_depth_mix(float*, const float*, int, long, int, const float*, void*, int, float, hipStream_t);
+int dllm_gelu_erf(const void*, void*, int, long, hipStream_t);
+int dllm_conv_refill(const void*, long, int, void*, int, int, const int*, const int*, const int*, const int*, int,
+                     hipStream_t);
+int dllm_delta_rule(const void*, long, const void*, long, int, int, int, int, int, const float*, const float*, const float*,
+                    float, float*, const int*, const int*, const int*, const int*, float*, void*, int, long, hipStream_t);
+int dllm_attn_prep(const void*, long, int, int, int, int, int, const float*, int, int, float, const float*, const int*,
+                   const int*, void*, void*, void*, long, hipStream_t);
+int dllm_gqa_tile_tokens(int, int);
+int dllm_paged_gqa(const void*, const void*, const void*, int, const int*, int, int, const int*, const int*, const int*,
+                   const int*, const int*, int, const void*, long, void*, int, int, int, int, hipStream_t);
 int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
 int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
 int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
@@ -1419,16 +1435,235 @@ void retention(torch::Tensor qkvg, int64_t H, int64_t d, int64_t dv, torch::Tens
     TORCH_CHECK(dllm_retention_chunk_lds((int)d) <= 150 * 1024, "dim does not fit the LDS");
     ok(dllm_retention_chunked(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, cos_sin.data_ptr<float>(),
                               (int)cos_sin.size(1), (int)rot, decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps,
-                              m.qstart, m.qlen, m.ctx, m.rows, raw->data_ptr<float>(), out.data_ptr(), m.S, (long)T,
-                              stream()),
+                              m.qstart, m.qlen, m.ctx, m.rows, raw->data_ptr<float>(), out.data_ptr(), m.S, (long)T, 0,
+                              1.f / std::sqrt((float)d), 1, stream()),
        "retention (chunked)");
     return;
   }
   TORCH_CHECK(dllm_retention_lds((int)d, (int)dv) <= 150 * 1024, "dim x vdim state does not fit the LDS");
   ok(dllm_retention(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, cos_sin.data_ptr<float>(),
                     (int)cos_sin.size(1), (int)rot, decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps, m.qstart,
-                    m.qlen, m.ctx, m.rows, out.data_ptr(), m.S, stream()),
+                    m.qlen, m.ctx, m.rows, out.data_ptr(), m.S, 0, 1.f / std::sqrt((float)d), nullptr, stream()),
      "retention");
+}
+
+// Lightning attention on the retention kernels: SiLU'd q / k / v, no rotation, no key scale, raw f32
+// outputs [T, H, dv]; then the heads of a token are normed together and gated by a sigmoid.
+void lightning_attention(torch::Tensor qkvg, int64_t H, int64_t d, int64_t dv, torch::Tensor decay, torch::Tensor state,
+                         double eps, torch::Tensor norm_w, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
+                         torch::Tensor rows, torch::Tensor out, torch::Tensor raw, bool chunked) {
+  const bool f = act_f32(qkvg, "qkvg");
+  check_rows2d(qkvg, "qkvg");
+  check_f32(decay, "decay");
+  check_f32(state, "state");
+  check_f32(norm_w, "norm weight");
+  check_f32(raw, "raw");
+  const int T = qkvg.size(0);
+  TORCH_CHECK(H >= 1 && d >= 1 && dv >= 1 && qkvg.size(1) >= 2 * H * d + 2 * H * dv, "qkvg [T, 2 H d + 2 H dv]");
+  TORCH_CHECK(decay.numel() == H && norm_w.numel() == H * dv, "decay per head, norm weight [H dv]");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == d && state.size(3) == dv,
+              "state [slots, H, d, dv]");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == qkvg.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == H * dv,
+              "out [T, H dv]");
+  TORCH_CHECK(raw.numel() >= (int64_t)T * H * dv, "raw scratch [T, H, dv]");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  if (chunked) {
+    TORCH_CHECK(dllm_retention_chunk_lds((int)d) <= 150 * 1024, "dim does not fit the LDS");
+    ok(dllm_retention_chunked(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, decay.data_ptr<float>(), 0, 0,
+                              decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps, m.qstart, m.qlen, m.ctx, m.rows,
+                              raw.data_ptr<float>(), out.data_ptr(), m.S, (long)T, 1, 1.f, 0, stream()),
+       "lightning attention (chunked)");
+  } else {
+    TORCH_CHECK(dllm_retention_lds((int)d, (int)dv) <= 150 * 1024, "dim x vdim state does not fit the LDS");
+    ok(dllm_retention(qkvg.data_ptr(), qkvg.stride(0), f, (int)H, (int)d, (int)dv, decay.data_ptr<float>(), 0, 0,
+                      decay.data_ptr<float>(), state.data_ptr<float>(), (float)eps, m.qstart, m.qlen, m.ctx, m.rows,
+                      out.data_ptr(), m.S, 1, 1.f, raw.data_ptr<float>(), stream()),
+       "lightning attention");
+  }
+  ok(dllm_heads_norm_gate(raw.data_ptr<float>(), qkvg.data_ptr(), qkvg.stride(0), f, 2 * H * d + H * dv, (int)(H * dv),
+                          norm_w.data_ptr<float>(), (float)eps, m.qstart, m.qlen, m.S, out.data_ptr(), (long)T, stream()),
+     "heads_norm_gate");
+}
+
+void resadd_norm(torch::Tensor a, c10::optional<torch::Tensor> b, c10::optional<torch::Tensor> wa,
+                 c10::optional<torch::Tensor> wb, torch::Tensor w_post, double eps, torch::Tensor x,
+                 c10::optional<torch::Tensor> w_next, c10::optional<torch::Tensor> xn) {
+  const bool f = act_f32(a, "a");
+  check_rows2d(a, "a");
+  check_f32(w_post, "w_post");
+  check_f32(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && x.sizes() == a.sizes() && w_post.numel() == x.size(1),
+              "x / a / w_post shapes");
+  const void* bp = nullptr;
+  const float *wap = nullptr, *wbp = nullptr, *wnp = nullptr;
+  long ldb = 0;
+  if (b) {
+    TORCH_CHECK(wa && wb, "two branches need both norm weights");
+    check_rows2d(*b, "b");
+    check_f32(*wa, "wa");
+    check_f32(*wb, "wb");
+    TORCH_CHECK(b->is_cuda() && b->scalar_type() == a.scalar_type() && b->sizes() == a.sizes() &&
+                    wa->numel() == x.size(1) && wb->numel() == x.size(1),
+                "b / wa / wb shapes");
+    bp = b->data_ptr();
+    ldb = b->stride(0);
+    wap = wa->data_ptr<float>();
+    wbp = wb->data_ptr<float>();
+  }
+  void* xp = nullptr;
+  if (xn) {
+    TORCH_CHECK(xn->is_cuda() && xn->scalar_type() == a.scalar_type() && xn->is_contiguous() && xn->sizes() == x.sizes(),
+                "x_next: contiguous, the dtype of a, the shape of x");
+    xp = xn->data_ptr();
+    if (w_next) {
+      check_f32(*w_next, "w_next");
+      TORCH_CHECK(w_next->numel() == x.size(1), "w_next length");
+      wnp = w_next->data_ptr<float>();
+    }
+  }
+  ok(dllm_resadd_norm(a.data_ptr(), a.stride(0), bp, ldb, f, wap, wbp, w_post.data_ptr<float>(), x.data_ptr<float>(), wnp,
+                      xp, (int)x.size(0), (int)x.size(1), (float)eps, stream()),
+     "resadd_norm");
+}
+
+void depth_mix(torch::Tensor X, torch::Tensor w, int64_t n, c10::optional<torch::Tensor> w_next, double eps,
+               c10::optional<torch::Tensor> xn) {
+  check_f32(X, "X");
+  check_f32(w, "w");
+  TORCH_CHECK(X.dim() == 3 && X.is_contiguous() && n >= 1 && n < X.size(0) && w.numel() >= n, "X [slots, T, H], n < slots");
+  void* xp = nullptr;
+  const float* wnp = nullptr;
+  bool f = true;
+  if (xn) {
+    f = act_f32(*xn, "out_next");
+    TORCH_CHECK(xn->is_contiguous() && xn->dim() == 2 && xn->size(0) == X.size(1) && xn->size(1) == X.size(2), "out_next [T, H]");
+    xp = xn->data_ptr();
+    if (w_next) {
+      check_f32(*w_next, "w_next");
+      TORCH_CHECK(w_next->numel() == X.size(2), "w_next length");
+      wnp = w_next->data_ptr<float>();
+    }
+  }
+  ok(dllm_depth_mix(X.data_ptr<float>(), w.data_ptr<float>(), (int)n, X.size(1), (int)X.size(2), wnp, xp, f, (float)eps,
+                    stream()),
+     "depth_mix");
+}
+
+void gelu_erf(torch::Tensor x, torch::Tensor y) {
+  const bool f = act_f32(x, "x");
+  TORCH_CHECK(x.is_contiguous() && y.is_cuda() && y.is_contiguous() && y.scalar_type() == x.scalar_type() &&
+                  y.sizes() == x.sizes(),
+              "x / y contiguous, same dtype and shape");
+  ok(dllm_gelu_erf(x.data_ptr(), y.data_ptr(), f, x.numel(), stream()), "gelu_erf");
+}
+
+void conv_state_refill(torch::Tensor x, torch::Tensor state, torch::Tensor qstart, torch::Tensor qlen, torch::Tensor ctx,
+                       torch::Tensor rows) {
+  const bool f = act_f32(x, "x");
+  check_rows2d(x, "x");
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == x.scalar_type() && state.is_contiguous() && state.dim() == 3 &&
+                  state.size(2) <= x.size(1) && state.size(1) <= 8,
+              "conv state [slots, taps - 1 <= 8, C <= columns of x]");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  ok(dllm_conv_refill(x.data_ptr(), x.stride(0), f, state.data_ptr(), (int)state.size(1), (int)state.size(2), m.qstart, m.qlen,
+                      m.ctx, m.rows, m.S, stream()),
+     "conv_state_refill");
+}
+
+void delta_rule(torch::Tensor qkv, torch::Tensor gba, int64_t H, int64_t G, int64_t d, int64_t dv, torch::Tensor neg_a,
+                torch::Tensor dt_bias, torch::Tensor norm_w, double eps, torch::Tensor state, torch::Tensor qstart,
+                torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor out) {
+  const bool f = act_f32(qkv, "qkv");
+  check_rows2d(qkv, "qkv");
+  check_rows2d(gba, "gba");
+  check_f32(neg_a, "neg_a");
+  check_f32(dt_bias, "dt_bias");
+  check_f32(norm_w, "norm weight");
+  check_f32(state, "state");
+  const int64_t T = qkv.size(0);
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && d >= 1 && d <= 256 && dv >= 1, "heads / kv_heads / dim <= 256 / vdim");
+  TORCH_CHECK(qkv.size(1) >= 2 * G * d + H * dv, "qkv [T, 2 G d + H dv]");
+  TORCH_CHECK(gba.is_cuda() && gba.scalar_type() == qkv.scalar_type() && gba.size(0) == T && gba.size(1) >= H * dv + 2 * H,
+              "gba [T, H dv + 2 H]");
+  TORCH_CHECK(neg_a.numel() == H && dt_bias.numel() == H && norm_w.numel() == dv, "per-head constants, norm weight [dv]");
+  TORCH_CHECK(state.dim() == 4 && state.is_contiguous() && state.size(1) == H && state.size(2) == dv && state.size(3) == d,
+              "state [slots, H, dv, d]");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == qkv.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == H * dv,
+              "out [T, H dv]");
+  auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
+  auto raw = torch::zeros({T, H, dv}, torch::TensorOptions().dtype(torch::kFloat32).device(qkv.device()));
+  ok(dllm_delta_rule(qkv.data_ptr(), qkv.stride(0), gba.data_ptr(), gba.stride(0), f, (int)H, (int)G, (int)d, (int)dv,
+                     neg_a.data_ptr<float>(), dt_bias.data_ptr<float>(), norm_w.data_ptr<float>(), (float)eps,
+                     state.data_ptr<float>(), m.qstart, m.qlen, m.ctx, m.rows, raw.data_ptr<float>(), out.data_ptr(), m.S,
+                     (long)T, stream()),
+     "delta_rule");
+}
+
+void attn_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, torch::Tensor cos_sin, int64_t rot,
+               double eps, torch::Tensor qscale, torch::Tensor pos, torch::Tensor slots, torch::Tensor kc, torch::Tensor vc,
+               torch::Tensor q) {
+  const bool f = act_f32(proj, "proj");
+  check_rows2d(proj, "proj");
+  check_f32(cos_sin, "cos_sin");
+  check_f32(qscale, "qscale");
+  check_i32(pos, "positions");
+  check_i32(slots, "slots");
+  const int64_t T = proj.size(0);
+  TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && proj.size(1) >= (H + G) * d + G * dv, "proj [T, (H + G) d + G dv]");
+  TORCH_CHECK(cos_sin.dim() == 2 && rot >= 0 && rot % 2 == 0 && rot <= d && (rot == 0 || cos_sin.size(1) >= rot),
+              "rotation table");
+  TORCH_CHECK(qscale.numel() == H && pos.numel() == T && slots.numel() == T, "qscale / positions / slots lengths");
+  for (auto* c : {&kc, &vc})
+    TORCH_CHECK(c->is_cuda() && c->scalar_type() == proj.scalar_type() && c->is_contiguous() && c->dim() == 4 &&
+                    c->size(2) == G,
+                "paged cache [blocks, block, G, width] in the activations' dtype");
+  TORCH_CHECK(kc.size(3) == d && vc.size(3) == dv && kc.size(0) == vc.size(0) && kc.size(1) == vc.size(1), "cache widths");
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == proj.scalar_type() && q.is_contiguous() && q.numel() == T * H * d, "q [T, H, d]");
+  ok(dllm_attn_prep(proj.data_ptr(), proj.stride(0), f, (int)H, (int)G, (int)d, (int)dv, cos_sin.data_ptr<float>(),
+                    (int)cos_sin.size(1), (int)rot, (float)eps, qscale.data_ptr<float>(), pos.data_ptr<int>(),
+                    slots.data_ptr<int>(), kc.data_ptr(), vc.data_ptr(), q.data_ptr(), (long)T, stream()),
+     "attn_prep");
+}
+
+void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, torch::Tensor bt, torch::Tensor qstart,
+                         torch::Tensor qlen, torch::Tensor ctx, torch::Tensor tile_seq, torch::Tensor tile_tok0,
+                         c10::optional<torch::Tensor> gate, torch::Tensor out) {
+  const bool f = act_f32(q, "q");
+  TORCH_CHECK(q.dim() == 3 && q.is_contiguous(), "q [T, H, d]");
+  const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
+  for (auto* c : {&kc, &vc})
+    TORCH_CHECK(c->is_cuda() && c->scalar_type() == q.scalar_type() && c->is_contiguous() && c->dim() == 4,
+                "paged cache [blocks, block, G, width] in the dtype of q");
+  const int64_t G = kc.size(2), dv = vc.size(3);
+  TORCH_CHECK(G >= 1 && H % G == 0 && kc.size(3) == d && vc.size(2) == G && kc.size(0) == vc.size(0) &&
+                  kc.size(1) == vc.size(1) && dv <= 256,
+              "cache shapes; vdim <= 256");
+  check_i32(bt, "block_tables");
+  TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1, "block_tables [S, blocks]");
+  for (auto* t : {&qstart, &qlen, &ctx, &tile_seq, &tile_tok0}) check_i32(*t, "sequence / tile metadata");
+  TORCH_CHECK(qlen.numel() == qstart.numel() && ctx.numel() == qstart.numel() && tile_tok0.numel() >= tile_seq.numel() &&
+                  bt.size(0) >= qstart.numel(),
+              "metadata lengths");
+  const void* gp = nullptr;
+  long ldg = 0;
+  if (gate) {
+    check_rows2d(*gate, "gate");
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == q.scalar_type() && gate->size(0) == T && gate->size(1) == H * dv,
+                "gate [T, H dv]");
+    gp = gate->data_ptr();
+    ldg = gate->stride(0);
+  }
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == q.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
+                  out.size(0) == T && out.size(1) == H * dv,
+              "out [T, H dv]");
+  const int rc = dllm_paged_gqa(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), f, bt.data_ptr<int>(), (int)bt.stride(0),
+                                (int)kc.size(1), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
+                                tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), gp, ldg,
+                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, stream());
+  TORCH_CHECK(rc != -2, "head widths do not fit the LDS");
+  ok(rc, "paged_gqa_attention");
 }
 
 void relu2_scale(torch::Tensor x, c10::optional<torch::Tensor> gate, int64_t ff, torch::Tensor y) {
@@ -1538,6 +1773,15 @@ PYBIND11_MODULE(_hip_kernels, m) {
         py::arg("qlen"), py::arg("ctx"), py::arg("rows"), py::arg("out"), py::arg("raw") = py::none());
   m.def("relu2_scale", &relu2_scale);
   m.def("dense_gate", &dense_gate);
+  m.def("lightning_attention", &lightning_attention);
+  m.def("resadd_norm", &resadd_norm);
+  m.def("depth_mix", &depth_mix);
+  m.def("gelu_erf", &gelu_erf);
+  m.def("conv_state_refill", &conv_state_refill);
+  m.def("delta_rule", &delta_rule);
+  m.def("attn_prep", &attn_prep);
+  m.def("paged_gqa_attention", &paged_gqa_attention);
+  m.def("gqa_tile_tokens", [](int64_t H, int64_t G) { return (int64_t)dllm_gqa_tile_tokens((int)H, (int)G); });
   m.def("latent_kv_write", &latent_kv_write);
   m.def("latent_attention", &latent_attention, py::arg("qa"), py::arg("q"), py::arg("dim"), py::arg("rot"),
         py::arg("positions"), py::arg("cos_sin"), py::arg("cache"), py::arg("block_tables"), py::arg("qstart"),

@@ -13,6 +13,9 @@
 //   retention_chunk  the same recurrence for prompt portions in its chunked form (32 tokens at a time:
 //                    scores inside the chunk + the carried state), one workgroup per (head, 32 value
 //                    columns, sequence); retention_finish norms and gates
+//   resadd_norm      x (f32) += rmsnorm(y) * w with y one branch or the normed average of two, plus the
+//                    next sublayer's normed input; depth_mix: a weighted sum over the f32 stack of
+//                    layer results, plus the normed input of the next layer; gelu_erf; conv_refill
 //   relu2_scale      relu(x)^2 (* a per-(token, expert) gate): squared-ReLU experts, dense form
 //   dense_gate       top-k (id, weight) pairs -> [T, E] gate matrix
 //
@@ -63,6 +66,106 @@ __global__ void __launch_bounds__(256) norm_resadd_kernel(const T* __restrict__ 
     xr[i] = v;
     if (xl) stf(xl + row * (long)H + i, v);
   }
+}
+
+// ---------------------------------------------------------------- resadd_norm, depth_mix, gelu
+// The tail of a sublayer whose output is normed before the add, and the norm ahead of the next
+// sublayer, for one token per workgroup:
+//   y = a                                        (one branch)
+//   y = (rmsnorm(a) wa + rmsnorm(b) wb) / 2      (two mixers side by side)
+//   x += rmsnorm(y) w_post;  xn = rmsnorm(x) w_next  (xn = x rounded when w_next is null)
+template <typename T>
+__global__ void __launch_bounds__(256) resadd_norm_kernel(const T* __restrict__ a, long lda, const T* __restrict__ b,
+                                                          long ldb, const float* __restrict__ wa,
+                                                          const float* __restrict__ wb, const float* __restrict__ w_post,
+                                                          float* __restrict__ x, const float* __restrict__ w_next,
+                                                          T* __restrict__ xn, int H, float eps) {
+  __shared__ float red[16];
+  extern __shared__ float yb[];   // [H]; entry i is touched by thread i % 256 only
+  const long row = blockIdx.x;
+  const T* ar = a + row * lda;
+  const T* br = b ? b + row * ldb : nullptr;
+  float ra = 1.f, rb = 1.f;
+  if (br) {
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+      const float va = ldf(ar + i), vb = ldf(br + i);
+      sa += va * va;
+      sb += vb * vb;
+    }
+    ra = 1.f / sqrtf(block_sum(sa, red) / (float)H + eps);
+    rb = 1.f / sqrtf(block_sum(sb, red) / (float)H + eps);
+  }
+  float sy = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float y = ldf(ar + i);
+    if (br) y = 0.5f * (y * ra * wa[i] + ldf(br + i) * rb * wb[i]);
+    yb[i] = y;
+    sy += y * y;
+  }
+  const float ry = 1.f / sqrtf(block_sum(sy, red) / (float)H + eps);
+  float* xr = x + row * (long)H;
+  float sx = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float v = xr[i] + yb[i] * ry * w_post[i];
+    xr[i] = v;
+    yb[i] = v;
+    sx += v * v;
+  }
+  if (!xn) return;
+  float rx = 1.f;
+  if (w_next) rx = 1.f / sqrtf(block_sum(sx, red) / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) stf(xn + row * (long)H + i, w_next ? yb[i] * rx * w_next[i] : yb[i]);
+}
+
+// X[n] = sum_{j<n} w[j] X[j] for one token per workgroup (X [slots][T][H] f32), xn = rmsnorm(X[n]) w_next
+template <typename T>
+__global__ void __launch_bounds__(256) depth_mix_kernel(float* __restrict__ X, const float* __restrict__ w, int n, long TH,
+                                                        const float* __restrict__ w_next, T* __restrict__ xn, int H,
+                                                        float eps) {
+  __shared__ float red[16];
+  extern __shared__ float yb[];
+  const long row = blockIdx.x;
+  float sx = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float* p = X + row * (long)H + i;
+    float acc = 0.f;
+    for (int j = 0; j < n; ++j) acc += w[j] * p[j * TH];
+    X[n * TH + row * (long)H + i] = acc;
+    yb[i] = acc;
+    sx += acc * acc;
+  }
+  if (!xn) return;
+  float rx = 1.f;
+  if (w_next) rx = 1.f / sqrtf(block_sum(sx, red) / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) stf(xn + row * (long)H + i, w_next ? yb[i] * rx * w_next[i] : yb[i]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) gelu_erf_kernel(const T* __restrict__ x, T* __restrict__ y, long n) {
+  for (long e = (long)blockIdx.x * 256 + threadIdx.x; e < n; e += (long)gridDim.x * 256) {
+    const float v = ldf(x + e);
+    stf(y + e, 0.5f * v * (1.f + erff(v * 0.70710678118654752f)));
+  }
+}
+
+// the last K - 1 inputs of every sequence go to its slot (read before they are overwritten)
+template <typename T>
+__global__ void __launch_bounds__(256) conv_refill_kernel(const T* __restrict__ x, long ldx, T* __restrict__ conv, int Km1,
+                                                          int C, const int* __restrict__ qstart,
+                                                          const int* __restrict__ qlen, const int* __restrict__ ctx,
+                                                          const int* __restrict__ rows) {
+  const int s = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  const int n = qlen[s];
+  if (n <= 0 || c >= C) return;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  T* cs = conv + (long)rows[s] * Km1 * C + c;
+  float u[8];
+  for (int k = 0; k < Km1; ++k) {
+    const int i = n - Km1 + k;
+    u[k] = i >= 0 ? ldf(x + (long)(q0 + i) * ldx + c) : (p0 > 0 ? ldf(cs + (long)(Km1 + i) * C) : 0.f);
+  }
+  for (int k = 0; k < Km1; ++k) stf(cs + (long)k * C, u[k]);
 }
 
 // ---------------------------------------------------------------- causal conv + SiLU
@@ -206,7 +309,8 @@ __global__ void __launch_bounds__(256) retention_kernel(const T* __restrict__ qk
                                                         const float* __restrict__ decay, float* __restrict__ state,
                                                         float eps, const int* __restrict__ qstart,
                                                         const int* __restrict__ qlen, const int* __restrict__ ctx,
-                                                        const int* __restrict__ rows, T* __restrict__ out, int LJ) {
+                                                        const int* __restrict__ rows, T* __restrict__ out, int LJ,
+                                                        int act, float kscale, float* __restrict__ raw) {
   extern __shared__ float sm[];
   const int h = blockIdx.x, s = blockIdx.y;
   const int n = qlen[s];
@@ -222,7 +326,7 @@ __global__ void __launch_bounds__(256) retention_kernel(const T* __restrict__ qk
   const int tid = threadIdx.x, j0 = tid % LJ, g = tid / LJ;
   float* sg = state + ((long)rows[s] * H + h) * d * dv;
   for (int e = tid; e < d * dv; e += 256) S[e] = p0 > 0 ? sg[e] : 0.f;
-  const float dec = decay[h], kscale = 1.f / sqrtf((float)d);
+  const float dec = decay[h];
   const int half = rot >> 1;
   const long oq = (long)h * d, ok = (long)H * d + (long)h * d, ov = 2L * H * d + (long)h * dv,
              og = 2L * H * d + (long)H * dv + (long)h * dv;
@@ -244,12 +348,14 @@ __global__ void __launch_bounds__(256) retention_kernel(const T* __restrict__ qk
         qv = i < half ? qv * c - qp * sn : qv * c + qp * sn;
         kv = i < half ? kv * c - kp * sn : kv * c + kp * sn;
       }
+      if (act) { qv = silu_f(qv); kv = silu_f(kv); }
       qs[e] = qv;
       ks[e] = kv * kscale;
     }
     for (int e = tid; e < nt * dv; e += 256) {
       const int tt = e / dv, j = e % dv;
-      vs[e] = ldf(qkvg + (long)(q0 + t0 + tt) * ld + ov + j);
+      const float vv = ldf(qkvg + (long)(q0 + t0 + tt) * ld + ov + j);
+      vs[e] = act ? silu_f(vv) : vv;
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
@@ -274,6 +380,13 @@ __global__ void __launch_bounds__(256) retention_kernel(const T* __restrict__ qk
       buf ^= 1;
     }
     __syncthreads();
+    if (raw) {   // the caller norms and gates (heads normed together)
+      for (int e = tid; e < nt * dv; e += 256) {
+        const int tt = e / dv, j = e % dv;
+        raw[((long)(q0 + t0 + tt) * H + h) * dv + j] = os[e];
+      }
+      continue;
+    }
     // unit-RMS head, SiLU gate, store: one wave per token
     for (int tt = tid >> 6; tt < nt; tt += 4) {
       const int lane = tid & 63;
@@ -307,7 +420,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restric
                                                               const float* __restrict__ decay, float* __restrict__ state,
                                                               const int* __restrict__ qstart, const int* __restrict__ qlen,
                                                               const int* __restrict__ ctx, const int* __restrict__ rows,
-                                                              float* __restrict__ raw) {
+                                                              float* __restrict__ raw, int act, float kscale) {
   extern __shared__ float sm[];
   const int h = blockIdx.x, v0 = blockIdx.y * RC_V, s = blockIdx.z;
   const int n = qlen[s];
@@ -326,7 +439,7 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restric
     const int i = e / RC_V, j = e % RC_V;
     S[e] = (p0 > 0 && j < nv) ? sg[(long)i * dv + v0 + j] : 0.f;
   }
-  const float dec = decay[h], kscale = 1.f / sqrtf((float)d);
+  const float dec = decay[h];
   if (tid <= RC_T) gp[tid] = powf(dec, (float)tid);
   const int half = rot >> 1;
   const long oq = (long)h * d, ok = (long)H * d + (long)h * d, ov = 2L * H * d + (long)h * dv + v0;
@@ -349,13 +462,15 @@ __global__ void __launch_bounds__(256) retention_chunk_kernel(const T* __restric
           qv = i < half ? qv * c - qp * sn : qv * c + qp * sn;
           kv = i < half ? kv * c - kp * sn : kv * c + kp * sn;
         }
+        if (act) { qv = silu_f(qv); kv = silu_f(kv); }
       }
       Qs[tt * dp + i] = qv;
       Ks[tt * dp + i] = kv * kscale;
     }
     for (int e = tid; e < RC_T * RC_V; e += 256) {
       const int tt = e / RC_V, j = e % RC_V;
-      Vs[e] = (tt < nt && j < nv) ? ldf(qkvg + (long)(q0 + t0 + tt) * ld + ov + j) : 0.f;
+      float vv = (tt < nt && j < nv) ? ldf(qkvg + (long)(q0 + t0 + tt) * ld + ov + j) : 0.f;
+      Vs[e] = act ? silu_f(vv) : vv;
     }
     __syncthreads();
     // scores inside the chunk: thread (t, 4 keys u0..u0+3); one q read serves four sums
@@ -461,6 +576,28 @@ __global__ void __launch_bounds__(256) retention_finish_kernel(const float* __re
     stf(out + tok * ((long)H * dv) + (long)h * dv + j, o[j] * rs * silu_f(ldf(qkvg + tok * ld + og + j)));
 }
 
+// the heads of a token normed together (weight w over heads x dv), times sigmoid(gate): one
+// workgroup per token
+template <typename T>
+__global__ void __launch_bounds__(256) heads_norm_gate_kernel(const float* __restrict__ raw, const T* __restrict__ qkvg,
+                                                              long ld, long og, int n, const float* __restrict__ w,
+                                                              float eps, const int* __restrict__ qstart,
+                                                              const int* __restrict__ qlen, int S, T* __restrict__ out) {
+  __shared__ float red[16];
+  const long tok = blockIdx.x;
+  bool live = false;
+  for (int s = 0; s < S; ++s) live |= tok >= qstart[s] && tok < qstart[s] + qlen[s];
+  if (!live) return;     // the whole workgroup: rows of no sequence keep their zeros
+  const float* o = raw + tok * n;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < n; j += 256) ss += o[j] * o[j];
+  const float rs = 1.f / sqrtf(block_sum(ss, red) / (float)n + eps);
+  for (int j = threadIdx.x; j < n; j += 256) {
+    const float gz = ldf(qkvg + tok * ld + og + j);
+    stf(out + tok * n + j, o[j] * rs * w[j] / (1.f + expf(-gz)));
+  }
+}
+
 // ---------------------------------------------------------------- squared ReLU, dense gate
 template <typename T>
 __global__ void __launch_bounds__(256) relu2_kernel(const T* __restrict__ x, const float* __restrict__ gate, int E,
@@ -522,6 +659,60 @@ extern "C" int dllm_norm_resadd(const void* y, long ldy, int f32, const float* w
   return (int)hipGetLastError();
 }
 
+extern "C" int dllm_resadd_norm(const void* a, long lda, const void* b, long ldb, int f32, const float* wa, const float* wb,
+                                const float* w_post, float* x, const float* w_next, void* xn, int rows, int H, float eps,
+                                hipStream_t st) {
+  if (rows <= 0) return rows == 0 ? 0 : -1;
+  const long lds = 4L * H;
+  if (lds > 150 * 1024) return -2;
+  if (f32) {
+    ENSURE_LDS(resadd_norm_kernel<float>, lds);
+    hipLaunchKernelGGL(resadd_norm_kernel<float>, dim3(rows), dim3(256), lds, st, (const float*)a, lda, (const float*)b, ldb, wa,
+                       wb, w_post, x, w_next, (float*)xn, H, eps);
+  } else {
+    ENSURE_LDS(resadd_norm_kernel<u16>, lds);
+    hipLaunchKernelGGL(resadd_norm_kernel<u16>, dim3(rows), dim3(256), lds, st, (const u16*)a, lda, (const u16*)b, ldb, wa, wb,
+                       w_post, x, w_next, (u16*)xn, H, eps);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_depth_mix(float* X, const float* w, int n, long T, int H, const float* w_next, void* xn, int f32,
+                              float eps, hipStream_t st) {
+  if (T <= 0) return T == 0 ? 0 : -1;
+  const long lds = 4L * H;
+  if (lds > 150 * 1024) return -2;
+  if (f32) {
+    ENSURE_LDS(depth_mix_kernel<float>, lds);
+    hipLaunchKernelGGL(depth_mix_kernel<float>, dim3((unsigned)T), dim3(256), lds, st, X, w, n, T * H, w_next, (float*)xn, H, eps);
+  } else {
+    ENSURE_LDS(depth_mix_kernel<u16>, lds);
+    hipLaunchKernelGGL(depth_mix_kernel<u16>, dim3((unsigned)T), dim3(256), lds, st, X, w, n, T * H, w_next, (u16*)xn, H, eps);
+  }
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_gelu_erf(const void* x, void* y, int f32, long n, hipStream_t st) {
+  if (n <= 0) return 0;
+  long gr = (n + 255) / 256;
+  if (gr > 8192) gr = 8192;
+  BY_T(f32,
+       hipLaunchKernelGGL(gelu_erf_kernel<u16>, dim3((int)gr), dim3(256), 0, st, (const u16*)x, (u16*)y, n),
+       hipLaunchKernelGGL(gelu_erf_kernel<float>, dim3((int)gr), dim3(256), 0, st, (const float*)x, (float*)y, n))
+  return (int)hipGetLastError();
+}
+
+extern "C" int dllm_conv_refill(const void* x, long ldx, int f32, void* conv, int Km1, int C, const int* qstart,
+                                const int* qlen, const int* ctx, const int* rows, int S, hipStream_t st) {
+  if (S <= 0 || Km1 <= 0) return 0;
+  if (Km1 > 8) return -1;
+  const dim3 g((C + 255) / 256, S);
+  BY_T(f32,
+       hipLaunchKernelGGL(conv_refill_kernel<u16>, g, dim3(256), 0, st, (const u16*)x, ldx, (u16*)conv, Km1, C, qstart, qlen, ctx, rows),
+       hipLaunchKernelGGL(conv_refill_kernel<float>, g, dim3(256), 0, st, (const float*)x, ldx, (float*)conv, Km1, C, qstart, qlen, ctx, rows))
+  return (int)hipGetLastError();
+}
+
 extern "C" int dllm_conv_silu(const void* x, long ldx, int f32, const float* w, const float* b, const void* state,
                               const int* qstart, const int* qlen, const int* ctx, const int* rows, void* y, int T,
                               int S, int C, int K, hipStream_t st) {
@@ -572,7 +763,8 @@ extern "C" long dllm_retention_lds(int d, int dv) {
 
 extern "C" int dllm_retention(const void* qkvg, long ld, int f32, int H, int d, int dv, const float* cos_sin, int tab_w,
                               int rot, const float* decay, float* state, float eps, const int* qstart, const int* qlen,
-                              const int* ctx, const int* rows, void* out, int S, hipStream_t st) {
+                              const int* ctx, const int* rows, void* out, int S, int act, float kscale, float* raw,
+                              hipStream_t st) {
   if (S <= 0) return 0;
   if (rot < 0 || rot > d || (rot & 1) || rot > tab_w) return -1;
   const long lds = dllm_retention_lds(d, dv);
@@ -583,11 +775,11 @@ extern "C" int dllm_retention(const void* qkvg, long ld, int f32, int H, int d, 
   if (f32) {
     ENSURE_LDS(retention_kernel<float>, lds);
     hipLaunchKernelGGL(retention_kernel<float>, g, dim3(256), lds, st, (const float*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
-                       decay, state, eps, qstart, qlen, ctx, rows, (float*)out, lj);
+                       decay, state, eps, qstart, qlen, ctx, rows, (float*)out, lj, act, kscale, raw);
   } else {
     ENSURE_LDS(retention_kernel<u16>, lds);
     hipLaunchKernelGGL(retention_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
-                       decay, state, eps, qstart, qlen, ctx, rows, (u16*)out, lj);
+                       decay, state, eps, qstart, qlen, ctx, rows, (u16*)out, lj, act, kscale, raw);
   }
   return (int)hipGetLastError();
 }
@@ -600,7 +792,7 @@ extern "C" long dllm_retention_chunk_lds(int d) {
 extern "C" int dllm_retention_chunked(const void* qkvg, long ld, int f32, int H, int d, int dv, const float* cos_sin,
                                       int tab_w, int rot, const float* decay, float* state, float eps, const int* qstart,
                                       const int* qlen, const int* ctx, const int* rows, float* raw, void* out, int S,
-                                      long T, hipStream_t st) {
+                                      long T, int act, float kscale, int finish, hipStream_t st) {
   if (S <= 0 || T <= 0) return 0;
   if (rot < 0 || rot > d || (rot & 1) || rot > tab_w) return -1;
   const long lds = dllm_retention_chunk_lds(d);
@@ -611,16 +803,28 @@ extern "C" int dllm_retention_chunked(const void* qkvg, long ld, int f32, int H,
   if (f32) {
     ENSURE_LDS(retention_chunk_kernel<float>, lds);
     hipLaunchKernelGGL(retention_chunk_kernel<float>, g, dim3(256), lds, st, (const float*)qkvg, ld, H, d, dv, cos_sin, tab_w,
-                       rot, decay, state, qstart, qlen, ctx, rows, raw);
-    hipLaunchKernelGGL(retention_finish_kernel<float>, gf, dim3(256), 0, st, raw, (const float*)qkvg, ld, H, d, dv, eps, qstart,
+                       rot, decay, state, qstart, qlen, ctx, rows, raw, act, kscale);
+    if (finish) hipLaunchKernelGGL(retention_finish_kernel<float>, gf, dim3(256), 0, st, raw, (const float*)qkvg, ld, H, d, dv, eps, qstart,
                        qlen, S, (float*)out, rows_total);
   } else {
     ENSURE_LDS(retention_chunk_kernel<u16>, lds);
     hipLaunchKernelGGL(retention_chunk_kernel<u16>, g, dim3(256), lds, st, (const u16*)qkvg, ld, H, d, dv, cos_sin, tab_w, rot,
-                       decay, state, qstart, qlen, ctx, rows, raw);
-    hipLaunchKernelGGL(retention_finish_kernel<u16>, gf, dim3(256), 0, st, raw, (const u16*)qkvg, ld, H, d, dv, eps, qstart, qlen,
+                       decay, state, qstart, qlen, ctx, rows, raw, act, kscale);
+    if (finish) hipLaunchKernelGGL(retention_finish_kernel<u16>, gf, dim3(256), 0, st, raw, (const u16*)qkvg, ld, H, d, dv, eps, qstart, qlen,
                        S, (u16*)out, rows_total);
   }
+  return (int)hipGetLastError();
+}
+
+// raw [T, n] f32 (n = heads x dv) -> out = rmsnorm over n * w * sigmoid(gate); the gate is column
+// `og` onwards of qkvg
+extern "C" int dllm_heads_norm_gate(const float* raw, const void* qkvg, long ld, int f32, long og, int n, const float* w,
+                                    float eps, const int* qstart, const int* qlen, int S, void* out, long T,
+                                    hipStream_t st) {
+  if (S <= 0 || T <= 0) return 0;
+  BY_T(f32,
+       hipLaunchKernelGGL(heads_norm_gate_kernel<u16>, dim3((unsigned)T), dim3(256), 0, st, raw, (const u16*)qkvg, ld, og, n, w, eps, qstart, qlen, S, (u16*)out),
+       hipLaunchKernelGGL(heads_norm_gate_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, raw, (const float*)qkvg, ld, og, n, w, eps, qstart, qlen, S, (float*)out))
   return (int)hipGetLastError();
 }
 

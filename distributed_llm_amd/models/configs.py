@@ -88,8 +88,9 @@ def get_model_config(name: str, **overrides) -> ModelConfig:
 # ----------------------------------------------------------------------------- layer-list designs
 #
 # A hybrid design is a list of layers, each with a token mixer (state-space scan, retention, latent
-# attention) and an optional feed-forward; every size and constant comes from the model folder's
-# config.json.  ``family`` picks the model class (models.registry).
+# attention, gated delta rule, grouped-query softmax attention, lightning attention, or two of
+# them side by side) and an optional feed-forward; every size and constant comes from the model
+# folder's config.json.  ``family`` picks the model class (models.registry).
 
 @dataclass(frozen=True)
 class RopeSpec:
@@ -100,8 +101,11 @@ class RopeSpec:
 @dataclass(frozen=True)
 class MixerSpec:
     """One token mixer.  ``kind``: ``mamba1`` (inner, state, dt_rank, conv), ``retention`` (heads,
-    dim, vdim, decay per head, rot) or ``latent_attention`` (heads, dim, rot_dim, vdim, kv_rank,
-    q_rank, scale, rot)."""
+    dim, vdim, decay per head, rot), ``latent_attention`` (heads, dim, rot_dim, vdim, kv_rank,
+    q_rank, scale, rot), ``delta`` (gated delta rule: heads, kv_heads, dim, vdim, conv),
+    ``softmax_attention`` (grouped-query, paged: heads, kv_heads, dim, vdim, scale, rot),
+    ``lightning`` (heads, dim, vdim, decay per head) or ``parallel`` (``left`` and ``right`` mixers
+    over the same input)."""
     kind: str
     inner: int = 0
     state: int = 0
@@ -116,10 +120,21 @@ class MixerSpec:
     kv_rank: int = 0
     q_rank: int = 0
     scale: float = 1.0
+    kv_heads: int = 0
+    left: Optional["MixerSpec"] = None
+    right: Optional["MixerSpec"] = None
+
+    @property
+    def parts(self) -> Tuple["MixerSpec", ...]:
+        return (self.left, self.right) if self.kind == "parallel" else (self,)
 
     @property
     def recurrent(self) -> bool:
-        return self.kind in ("mamba1", "retention")
+        return any(p.kind in ("mamba1", "retention", "delta", "lightning") for p in self.parts)
+
+    @property
+    def paged(self) -> bool:
+        return any(p.kind in ("latent_attention", "softmax_attention") for p in self.parts)
 
 
 @dataclass(frozen=True)
@@ -134,9 +149,16 @@ class MoESpec:
 
 
 @dataclass(frozen=True)
+class DenseSpec:
+    """One dense feed-forward ``W_down act(W_up x)``, ``ff`` wide; ``act``: ``gelu`` (the erf form)."""
+    ff: int
+    act: str = "gelu"
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     mixer: MixerSpec
-    mlp: Optional[MoESpec] = None
+    mlp: Optional[Union[MoESpec, DenseSpec]] = None
 
 
 @dataclass(frozen=True)
@@ -151,6 +173,11 @@ class HybridConfig:
     max_position: int = 1 << 20       # the design has no position limit; the engine's max_model_len bounds it
     bos_id: int = 1
     eos_id: int = 2
+    # layer form.  False: x += norm(sublayer(x)).  True: x += norm_b(sublayer(norm(x))), a norm on
+    # both sides of every sublayer.
+    pre_norm: bool = False
+    # what a layer hands on is a learned weighted sum of the embedding output and every layer result so far
+    depth_average: bool = False
 
     @property
     def n_layers(self) -> int:
@@ -158,7 +185,7 @@ class HybridConfig:
 
     @property
     def is_moe(self) -> bool:
-        return any(L.mlp is not None for L in self.layers)
+        return any(isinstance(L.mlp, MoESpec) for L in self.layers)
 
     def num_params(self) -> int:
         H, n = self.hidden, 2 * self.vocab * self.hidden + self.hidden
@@ -167,15 +194,28 @@ class HybridConfig:
             if m.kind == "mamba1":
                 n += 2 * m.inner * H + m.inner * (m.conv + 1) + (m.dt_rank + 2 * m.state) * m.inner
                 n += m.inner * (m.dt_rank + 1) + m.inner * m.state + m.inner + H * m.inner
-            elif m.kind == "retention":
-                n += 2 * m.heads * m.dim * H + 2 * m.heads * m.vdim * H + H * m.heads * m.vdim
-            else:
-                n += m.q_rank * (H + 1) + m.heads * (m.dim + m.rot_dim) * m.q_rank + (m.kv_rank + m.rot_dim) * H
-                n += m.kv_rank + m.heads * (m.dim + m.vdim) * m.kv_rank + H * m.heads * m.vdim
-            n += H
-            if L.mlp is not None:
+            if m.kind == "parallel":
+                n += 2 * H      # each side's output norm
+            for m in L.mixer.parts:
+                if m.kind in ("retention", "lightning"):
+                    n += 2 * m.heads * m.dim * H + 2 * m.heads * m.vdim * H + H * m.heads * m.vdim
+                    n += m.heads * m.vdim if m.kind == "lightning" else 0
+                elif m.kind == "latent_attention":
+                    n += m.q_rank * (H + 1) + m.heads * (m.dim + m.rot_dim) * m.q_rank + (m.kv_rank + m.rot_dim) * H
+                    n += m.kv_rank + m.heads * (m.dim + m.vdim) * m.kv_rank + H * m.heads * m.vdim
+                elif m.kind == "softmax_attention":
+                    n += (m.heads + m.kv_heads) * m.dim * H + m.kv_heads * m.vdim * H + 2 * m.heads * m.vdim * H + m.heads
+                elif m.kind == "delta":
+                    c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
+                    n += c * (H + m.conv) + 2 * m.heads * (H + 1) + m.vdim + 2 * m.heads * m.vdim * H
+            n += H * (2 if self.pre_norm else 1)
+            if isinstance(L.mlp, MoESpec):
                 f = L.mlp
                 n += H + f.experts * (H + 2 * f.ff * H) + 2 * f.shared_ff * H
+            elif isinstance(L.mlp, DenseSpec):
+                n += 2 * H + 2 * L.mlp.ff * H
+        if self.depth_average:
+            n += sum(i + 2 for i in range(len(self.layers)))
         return n
 
 
@@ -214,8 +254,46 @@ def filevik_config(raw: dict, name: str = "filevik") -> HybridConfig:
                         rms_eps=float(raw["norm"]["eps"]), logit_scale=float(raw.get("logit_scale", 1.0)))
 
 
+def sedopel_config(raw: dict, name: str = "sedopel") -> HybridConfig:
+    """A Sedopel config.json: ``layers`` (type ``delta`` or ``parallel``, mixer sizes, mlp or null),
+    ``norm.eps``, ``vocab``, ``width``.  Every sublayer has a norm on both sides and every layer
+    ends in a weighted sum over depth."""
+    def attention(m: dict) -> MixerSpec:
+        return MixerSpec("softmax_attention", heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])),
+                         dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]), rot=_rope(m.get("rot")))
+
+    def lightning(m: dict) -> MixerSpec:
+        return MixerSpec("lightning", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                         decay=tuple(float(x) for x in m["decay"]))
+
+    layers = []
+    for L in raw["layers"]:
+        m, kind = L["mixer"], L["type"]
+        if kind == "delta":
+            mix = MixerSpec(kind, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                            vdim=int(m["vdim"]), conv=int(m["conv"]))
+        elif kind == "parallel":
+            mix = MixerSpec(kind, left=attention(m["left"]), right=lightning(m["right"]))
+        else:
+            raise ValueError(f"unknown mixer type {kind!r}")
+        for p in mix.parts:
+            if p.kv_heads and p.heads % p.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+            if p.kind == "lightning" and len(p.decay) != p.heads:
+                raise ValueError("one decay per head")
+        f = L.get("mlp")
+        mlp = None
+        if f:
+            if f.get("kind", "dense") != "dense":
+                raise ValueError(f"unknown feed-forward kind {f.get('kind')!r}")
+            mlp = DenseSpec(int(f["ff"]))
+        layers.append(LayerSpec(mix, mlp))
+    return HybridConfig(name, "sedopel", int(raw["width"]), int(raw["vocab"]), tuple(layers),
+                        rms_eps=float(raw["norm"]["eps"]), pre_norm=True, depth_average=True)
+
+
 # config.json "architecture" -> parser of that design's keys
-ARCHITECTURES = {"Filevik": filevik_config}
+ARCHITECTURES = {"Filevik": filevik_config, "Sedopel": sedopel_config}
 
 AnyConfig = Union[ModelConfig, HybridConfig]
 

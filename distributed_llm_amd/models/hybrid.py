@@ -1,5 +1,6 @@
-"""Layer-list decoder (Filevik): every layer has a token mixer (Mamba-1 selective scan, retention,
-latent attention) and an optional mixture-of-experts feed-forward, in the order config.json gives.
+"""Layer-list decoders (Filevik, Sedopel): every layer has a token mixer (Mamba-1 selective scan,
+retention, latent attention, gated delta rule, or grouped-query softmax attention beside lightning
+attention) and an optional feed-forward (mixture of experts or dense), in the order config.json gives.
 
 The residual stream lives in f32; each sublayer reads its rounding to the model dtype and adds
 ``rmsnorm(sublayer(x)) * w`` (ops.seqmix.norm_resadd: the f32 add, the norm and the rounded copy in
@@ -19,6 +20,19 @@ they do not take and for f32 models), everything between them on the HIP kernels
   experts    fused router (f32 softmax top-k, renormalised) -> grouped squared-ReLU expert GEMMs, or
              the dense form (all experts' columns, unused ones gated to zero) for f32 models and
              unaligned widths -> plus the shared expert
+  delta      one fused projection (q | k | v | gate | beta | decay logits) -> causal conv + SiLU ->
+             gated delta rule (unit q / k, decay, beta, f32 state per slot, per-head norm and SiLU
+             gate in the kernel) -> out-proj
+  parallel   one fused projection for both sides.  Left: rotation + unit-RMS q / k, k and v written
+             to their pages, causal softmax attention over the pages with the sigmoid gate ->
+             out-proj.  Right: lightning attention (the retention kernels on SiLU'd inputs, heads
+             normed together, sigmoid gate) -> out-proj.  The two outputs are normed and averaged
+             in the launch that also adds the sublayer to the stream.
+  dense      up-proj -> erf GELU -> down-proj
+
+Layer forms: ``x += norm(sublayer(x))`` (Filevik) or, with ``cfg.pre_norm``, a norm on both sides,
+``x += norm_b(sublayer(norm(x)))``; with ``cfg.depth_average`` a layer hands on a learned weighted
+sum of the embedding output and all layer results so far (kept as an f32 stack for the step).
 
 Per-sequence state lives in slots owned by the engine (its batch rows); paged latents use the
 engine's block tables.  No tensor parallelism.
@@ -35,7 +49,7 @@ import torch.nn.functional as F
 from .. import ops
 from ..ops import seqmix
 from ..parallel.comm import SINGLE, ParallelContext
-from .configs import HybridConfig, LayerSpec, MixerSpec, MoESpec
+from .configs import DenseSpec, HybridConfig, LayerSpec, MixerSpec, MoESpec
 
 
 def _mm(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -87,7 +101,31 @@ class HybridModel:
         for i, L in enumerate(cfg.layers):
             p, m = f"l{i}.", L.mixer
             t[p + "norm1"] = torch.ones(W)
-            if m.kind == "mamba1":
+            if cfg.pre_norm:
+                t[p + "norm1b"] = torch.ones(W)
+            if cfg.depth_average:
+                t[p + "dwa"] = torch.cat([rnd(i + 1, s=0.05), torch.ones(1)])
+            if m.kind == "delta":
+                gd, hv = m.kv_heads * m.dim, m.heads * m.vdim
+                for n_, c in (("q", gd), ("k", gd), ("v", hv)):
+                    t[p + "mix." + n_] = lin(c, W)
+                    t[p + f"mix.{n_}.conv"] = rnd(c, m.conv, s=1.0 / math.sqrt(m.conv))
+                t[p + "mix.g"], t[p + "mix.o"] = lin(hv, W), lin(W, hv)
+                t[p + "mix.b"], t[p + "mix.a"] = lin(m.heads, W), lin(m.heads, W)
+                t[p + "mix.A_log"] = torch.log(torch.rand(m.heads, generator=g) * 15 + 1)
+                dt = torch.exp(torch.rand(m.heads, generator=g) * (math.log(0.1) - math.log(0.001)) + math.log(0.001))
+                t[p + "mix.dt_bias"] = dt + torch.log(-torch.expm1(-dt))
+                t[p + "mix.norm"] = torch.ones(m.vdim)
+            elif m.kind == "parallel":
+                a, b = m.left, m.right
+                t[p + "mix.left.q"], t[p + "mix.left.k"] = lin(a.heads * a.dim, W), lin(a.kv_heads * a.dim, W)
+                t[p + "mix.left.v"], t[p + "mix.left.g"] = lin(a.kv_heads * a.vdim, W), lin(a.heads * a.vdim, W)
+                t[p + "mix.left.o"], t[p + "mix.left.temp"] = lin(W, a.heads * a.vdim), torch.ones(a.heads)
+                t[p + "mix.right.q"], t[p + "mix.right.k"] = lin(b.heads * b.dim, W), lin(b.heads * b.dim, W)
+                t[p + "mix.right.v"], t[p + "mix.right.g"] = lin(b.heads * b.vdim, W), lin(b.heads * b.vdim, W)
+                t[p + "mix.right.o"], t[p + "mix.right.norm"] = lin(W, b.heads * b.vdim), torch.ones(b.heads * b.vdim)
+                t[p + "mix.left.out"], t[p + "mix.right.out"] = torch.ones(W), torch.ones(W)
+            elif m.kind == "mamba1":
                 t[p + "mix.in"] = lin(2 * m.inner, W)
                 t[p + "mix.conv"] = rnd(m.inner, m.conv, s=1.0 / math.sqrt(m.conv))
                 t[p + "mix.conv.b"] = rnd(m.inner, s=0.1)
@@ -109,7 +147,12 @@ class HybridModel:
                 t[p + "mix.uk"], t[p + "mix.uv"] = lin(m.heads * m.dim, m.kv_rank), lin(m.heads * m.vdim, m.kv_rank)
                 t[p + "mix.o"] = lin(W, m.heads * m.vdim)
             f = L.mlp
-            if f is not None:
+            if isinstance(f, DenseSpec):
+                t[p + "norm2"] = torch.ones(W)
+                if cfg.pre_norm:
+                    t[p + "norm2b"] = torch.ones(W)
+                t[p + "mlp.up"], t[p + "mlp.down"] = lin(f.ff, W), lin(W, f.ff)
+            elif f is not None:
                 t[p + "norm2"] = torch.ones(W)
                 t[p + "mlp.router"] = lin(f.experts, W)
                 for e in range(f.experts):
@@ -143,7 +186,32 @@ class HybridModel:
         for i, L in enumerate(cfg.layers):
             p, m = f"l{i}.", L.mixer
             D: Dict[str, torch.Tensor] = {"norm1": f32(t[p + "norm1"])}
-            if m.kind == "mamba1":
+            if cfg.pre_norm:
+                D["norm1b"] = f32(t[p + "norm1b"])
+            if cfg.depth_average:
+                D["dwa"] = f32(t[p + "dwa"])
+                assert D["dwa"].numel() == i + 2
+            if m.kind == "delta":
+                # one projection: q | k | v (the convolved channels) | gate | beta | decay logits
+                D["proj"] = put(torch.cat([t[p + "mix." + n] for n in ("q", "k", "v", "g", "b", "a")], 0))
+                D["conv"] = f32(torch.cat([t[p + f"mix.{n}.conv"] for n in "qkv"], 0))
+                D["conv_b"] = torch.zeros(D["conv"].shape[0], dtype=torch.float32, device=dev)
+                D["neg_a"], D["dt_b"] = -torch.exp(f32(t[p + "mix.A_log"])), f32(t[p + "mix.dt_bias"])
+                D["hnorm"], D["o"] = f32(t[p + "mix.norm"]), put(t[p + "mix.o"])
+                assert tuple(D["conv"].shape) == (2 * m.kv_heads * m.dim + m.heads * m.vdim, m.conv)
+                assert D["neg_a"].numel() == m.heads and D["hnorm"].numel() == m.vdim
+            elif m.kind == "parallel":
+                a, b = m.left, m.right
+                names = [f"mix.left.{n}" for n in "qkvg"] + [f"mix.right.{n}" for n in "qkvg"]
+                D["proj"] = put(torch.cat([t[p + n] for n in names], 0))
+                D["lo"], D["ro"] = put(t[p + "mix.left.o"]), put(t[p + "mix.right.o"])
+                D["qscale"] = f32(t[p + "mix.left.temp"]) * a.scale
+                D["decay"] = torch.tensor(b.decay, dtype=torch.float32, device=dev)
+                D["rnorm"] = f32(t[p + "mix.right.norm"])
+                D["lout"], D["rout"] = f32(t[p + "mix.left.out"]), f32(t[p + "mix.right.out"])
+                assert D["qscale"].numel() == a.heads and D["rnorm"].numel() == b.heads * b.vdim
+                assert D["proj"].shape[0] == self._left_cols(a) + 2 * b.heads * (b.dim + b.vdim)
+            elif m.kind == "mamba1":
                 D["in"], D["x"], D["dt"], D["o"] = (put(t[p + "mix." + n]) for n in ("in", "x", "dt", "o"))
                 D["conv"], D["conv_b"] = f32(t[p + "mix.conv"]), f32(t[p + "mix.conv.b"])
                 D["dt_b"], D["D"] = f32(t[p + "mix.dt.b"]), f32(t[p + "mix.D"])
@@ -161,7 +229,12 @@ class HybridModel:
                 D["uk"] = put(t[p + "mix.uk"].view(m.heads, m.dim, m.kv_rank))                       # [H, d, r]
                 D["uvT"] = put(t[p + "mix.uv"].view(m.heads, m.vdim, m.kv_rank).transpose(1, 2))    # [H, r, dv]
             f = L.mlp
-            if f is not None:
+            if isinstance(f, DenseSpec):
+                D["norm2"], D["up"], D["down"] = f32(t[p + "norm2"]), put(t[p + "mlp.up"]), put(t[p + "mlp.down"])
+                if cfg.pre_norm:
+                    D["norm2b"] = f32(t[p + "norm2b"])
+                assert tuple(D["up"].shape) == (f.ff, W)
+            elif f is not None:
                 D["norm2"] = f32(t[p + "norm2"])
                 D["router"] = put(t[p + "mlp.router"])
                 w1 = torch.stack([t[p + f"mlp.e{e}.up"] for e in range(f.experts)])       # [E, ff, W]
@@ -187,7 +260,7 @@ class HybridModel:
         for L, S in zip(self.layers, self.cfg.layers):
             for k, x in L.items():
                 b = x.numel() * x.element_size()
-                if k in ("w1", "w2", "w2d") and top_only and S.mlp is not None:
+                if k in ("w1", "w2", "w2d") and top_only and isinstance(S.mlp, MoESpec):
                     b = b * S.mlp.top // S.mlp.experts
                 n += b
         return n
@@ -199,9 +272,10 @@ class HybridModel:
             return
         self._max_pos = n
         for L in self.cfg.layers:
-            r = L.mixer.rot
-            if r is not None and r.dims > 0:
-                self._rot[(r.dims, r.base)] = ops.rope_cos_sin(n, r.dims, r.base, self.device)
+            for m in L.mixer.parts:
+                r = m.rot
+                if r is not None and r.dims > 0:
+                    self._rot[(r.dims, r.base)] = ops.rope_cos_sin(n, r.dims, r.base, self.device)
 
     def _table(self, m: MixerSpec) -> torch.Tensor:
         return self._rot[(m.rot.dims, m.rot.base)]
@@ -209,17 +283,34 @@ class HybridModel:
     def block_bytes(self, block_size: int) -> int:
         """Bytes of one paged block over all layers (latent attention layers only)."""
         it = torch.empty((), dtype=self.dtype).element_size()
-        return sum(block_size * (L.mixer.kv_rank + L.mixer.rot_dim) * it for L in self.cfg.layers
-                   if L.mixer.kind == "latent_attention")
+        n = 0
+        for L in self.cfg.layers:
+            for m in L.mixer.parts:
+                if m.kind == "latent_attention":
+                    n += block_size * (m.kv_rank + m.rot_dim) * it
+                elif m.kind == "softmax_attention":
+                    n += block_size * m.kv_heads * (m.dim + m.vdim) * it
+        return n
 
     def alloc_caches(self, num_blocks: int, block_size: int, slots: int) -> List[tuple]:
         """Per layer: (paged latent [blocks, block, rank + rot],) or the recurrent state of ``slots``
         sequences: (conv inputs [slots, taps - 1, inner], scan state [slots, inner, state] f32) /
-        (retention state [slots, heads, dim, vdim] f32,)."""
+        (retention state [slots, heads, dim, vdim] f32,) / delta: (conv inputs [slots, taps - 1,
+        q | k | v channels], state [slots, heads, vdim, dim] f32) / parallel: (paged keys [blocks,
+        block, kv_heads, dim], paged values [.., vdim], lightning state [slots, heads, dim, vdim] f32)."""
         dev, out = self.device, []
         for L in self.cfg.layers:
             m = L.mixer
-            if m.kind == "mamba1":
+            if m.kind == "delta":
+                c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
+                out.append((torch.zeros((slots, max(m.conv - 1, 0), c), dtype=self.dtype, device=dev),
+                            torch.zeros((slots, m.heads, m.vdim, m.dim), dtype=torch.float32, device=dev)))
+            elif m.kind == "parallel":
+                a, b = m.left, m.right
+                out.append((torch.zeros((num_blocks, block_size, a.kv_heads, a.dim), dtype=self.dtype, device=dev),
+                            torch.zeros((num_blocks, block_size, a.kv_heads, a.vdim), dtype=self.dtype, device=dev),
+                            torch.zeros((slots, b.heads, b.dim, b.vdim), dtype=torch.float32, device=dev)))
+            elif m.kind == "mamba1":
                 out.append((torch.zeros((slots, max(m.conv - 1, 0), m.inner), dtype=self.dtype, device=dev),
                             torch.zeros((slots, m.inner, m.state), dtype=torch.float32, device=dev)))
             elif m.kind == "retention":
@@ -271,6 +362,43 @@ class HybridModel:
         o = torch.bmm(lat, L["uvT"])                                    # [H, T, vdim]
         return _mm(o.transpose(0, 1).reshape(T, H * m.vdim), L["o"])
 
+    @staticmethod
+    def _left_cols(a: MixerSpec) -> int:
+        """Columns of the softmax side in the fused projection: q | k | v | gate."""
+        return (a.heads + a.kv_heads) * a.dim + a.kv_heads * a.vdim + a.heads * a.vdim
+
+    def _delta(self, L, m: MixerSpec, x, meta, cache):
+        conv_state, state = cache
+        rows = meta.state_rows
+        c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
+        proj = _mm(x, L["proj"])                                        # q | k | v | gate | beta | decay logits
+        qkv = seqmix.causal_conv_silu(proj, L["conv"], L["conv_b"], conv_state, meta.qstart, meta.qlen, meta.ctx, rows)
+        seqmix.conv_state_refill(proj, conv_state, meta.qstart, meta.qlen, meta.ctx, rows)
+        o = seqmix.delta_rule(qkv, proj[:, c:], m.heads, m.kv_heads, m.dim, m.vdim, L["neg_a"], L["dt_b"], L["hnorm"],
+                              self.cfg.rms_eps, state, meta.qstart, meta.qlen, meta.ctx, rows)
+        return _mm(o, L["o"])
+
+    def _parallel(self, L, m: MixerSpec, x, positions, meta, cache):
+        """Both sides' outputs, un-normed: the caller's residual launch norms and averages them."""
+        a, b, eps = m.left, m.right, self.cfg.rms_eps
+        k_cache, v_cache, state = cache
+        proj = _mm(x, L["proj"])
+        nl = self._left_cols(a)
+        rot = a.rot.dims if a.rot is not None else 0
+        table = self._table(a) if rot else self._any_table()
+        q = seqmix.attn_prep(proj, a.heads, a.kv_heads, a.dim, a.vdim, table, rot, eps, L["qscale"], positions,
+                             meta.slots, k_cache, v_cache)
+        ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(a.heads, a.kv_heads))
+        gate = proj[:, nl - a.heads * a.vdim:nl]
+        lo = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
+                                        gate)
+        ro = seqmix.lightning_attention(proj[:, nl:], b.heads, b.dim, b.vdim, L["decay"], state, eps, L["rnorm"],
+                                        meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
+        return _mm(lo, L["lo"]), _mm(ro, L["ro"])
+
+    def _dense(self, L, f: DenseSpec, x):
+        return _mm(seqmix.gelu_erf(_mm(x, L["up"])), L["down"])
+
     def _experts(self, L, f: MoESpec, x):
         if f.experts > 64 or f.top > 8:      # beyond the router kernels' register budget: library top-k
             val, ids = torch.topk(torch.softmax(F.linear(x.float(), L["router"].float()), -1), f.top, -1)
@@ -309,21 +437,64 @@ class HybridModel:
         else:
             x = self.embed.index_select(0, input_ids.long())
             xl = None
-        for L, S, cache in zip(self.layers, cfg.layers, kv_caches):
+        T, W, nL = x.shape[0], cfg.hidden, len(self.layers)
+        X = None
+        if cfg.depth_average:
+            # f32 stack of the embedding output and every layer's result; layer i works in place on
+            # slot i + 1, which the previous layer's weighted sum has filled with its input
+            X = torch.empty((nL + 2, T, W), dtype=torch.float32, device=x.device)
+            X[0].copy_(x)
+            X[1].copy_(x)
+            x = X[1]
+        h = None
+        if cfg.pre_norm:
+            h = seqmix.rms_rows(x, self.layers[0]["norm1"], eps, out_dtype=self.dtype)
+        for i, (L, S, cache) in enumerate(zip(self.layers, cfg.layers, kv_caches)):
             m = S.mixer
-            h = x if xl is None else xl
+            if not cfg.pre_norm:
+                h = x if xl is None else xl
             if m.kind == "mamba1":
                 y = self._mamba(L, m, h, meta, cache)
             elif m.kind == "retention":
                 y = self._retention(L, m, h, positions, meta, cache)
+            elif m.kind == "delta":
+                y = self._delta(L, m, h, meta, cache)
+            elif m.kind == "parallel":
+                y = self._parallel(L, m, h, positions, meta, cache)
             else:
                 y = self._latent(L, m, h, positions, meta, cache)
-            seqmix.norm_resadd(y, L["norm1"], eps, x, xl)
-            if S.mlp is not None:
-                y = self._experts(L, S.mlp, x if xl is None else xl)
-                seqmix.norm_resadd(y, L["norm2"], eps, x, xl)
+            if cfg.pre_norm:
+                # the sublayer's tail and the next sublayer's input norm in one launch
+                nxt = self.layers[i + 1]["norm1"] if i + 1 < nL else self.final_norm
+                pair = dict(b=y[1], wa=L["lout"], wb=L["rout"]) if isinstance(y, tuple) else {}
+                a = y[0] if isinstance(y, tuple) else y
+                if S.mlp is not None:
+                    h = torch.empty((T, W), dtype=self.dtype, device=x.device)
+                    seqmix.resadd_norm(a, L["norm1b"], eps, x, L["norm2"], h, **pair)
+                    y = self._dense(L, S.mlp, h) if isinstance(S.mlp, DenseSpec) else self._experts(L, S.mlp, h)
+                    a, pair, post = y, {}, L["norm2b"]
+                else:
+                    post = L["norm1b"]
+                if X is not None:
+                    seqmix.resadd_norm(a, post, eps, x, **pair)
+                    h = torch.empty((T, W), dtype=self.dtype, device=x.device)
+                    x = seqmix.depth_mix(X, L["dwa"], i + 2, nxt, eps, h)
+                else:
+                    h = torch.empty((T, W), dtype=self.dtype, device=x.device)
+                    seqmix.resadd_norm(a, post, eps, x, nxt, h, **pair)
+            else:
+                seqmix.norm_resadd(y, L["norm1"], eps, x, xl)
+                if S.mlp is not None:
+                    y = self._experts(L, S.mlp, x if xl is None else xl)
+                    seqmix.norm_resadd(y, L["norm2"], eps, x, xl)
+                if X is not None:
+                    x = seqmix.depth_mix(X, L["dwa"], i + 2)
+                    if xl is not None:
+                        xl.copy_(x)
             if self.tap is not None:
                 self.tap.append(x.clone())
+        if cfg.pre_norm:     # h is the final-normed stream of every row
+            return h if meta.all_last else h.index_select(0, meta.last_idx)
         sel = x if meta.all_last else x.index_select(0, meta.last_idx)
         return seqmix.rms_rows(sel, self.final_norm, eps, out_dtype=self.dtype)
 

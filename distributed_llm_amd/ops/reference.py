@@ -550,3 +550,157 @@ def dense_gate(ids, wts, E):
     g = torch.zeros((ids.shape[0], E), dtype=torch.float32, device=ids.device)
     g.scatter_(1, ids.long(), wts.float())
     return g
+
+
+# ----------------------------------------------------------------------------- pre/post-norm layers, depth average
+
+def resadd_norm(a, w_post, eps, x, w_next=None, x_next=None, b=None, wa=None, wb=None):
+    """x (f32 stream, in place) += rmsnorm(y) * w_post with y = a, or, with a second branch,
+    y = (rmsnorm(a) wa + rmsnorm(b) wb) / 2; ``x_next`` receives rmsnorm(x) * w_next (the plain
+    rounding of x when ``w_next`` is None)."""
+    y = a.float() if b is None else 0.5 * (rms_rows(a, wa, eps, torch.float32) + rms_rows(b, wb, eps, torch.float32))
+    x += rms_rows(y, w_post, eps, torch.float32)
+    if x_next is not None:
+        x_next.copy_(x if w_next is None else rms_rows(x, w_next, eps, torch.float32))
+    return x
+
+
+def depth_mix(X, w, n, w_next=None, eps=0.0, out_next=None):
+    """X[n] = sum over j < n of w[j] X[j] (X [slots, T, width] f32); ``out_next`` receives
+    rmsnorm(X[n]) * w_next."""
+    X[n] = torch.einsum("j,jtw->tw", w[:n].float(), X[:n])
+    if out_next is not None:
+        out_next.copy_(X[n] if w_next is None else rms_rows(X[n], w_next, eps, torch.float32))
+    return X[n]
+
+
+def gelu_erf(x):
+    return torch.nn.functional.gelu(x.float()).to(x.dtype)
+
+
+# ----------------------------------------------------------------------------- grouped-query attention, paged
+
+def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots, k_cache, v_cache):
+    """proj [T, >= heads dim + kv_heads (dim + vdim)] (q | k | v).  q and k: rotate-half positions on
+    the first ``rot_dims`` dims of each head, then each head to unit RMS; q times ``qscale[head]``.
+    k and v go to their page slots (k_cache [blocks, block, kv_heads, dim], v_cache [..., vdim]);
+    returns q [T, heads, dim]."""
+    T, H, G, d, dv = proj.shape[0], heads, kv_heads, dim, vdim
+    pf = proj.float()
+    q = pf[:, :H * d].reshape(T, H, d).clone()
+    k = pf[:, H * d:(H + G) * d].reshape(T, G, d).clone()
+    v = pf[:, (H + G) * d:(H + G) * d + G * dv].reshape(T, G, dv)
+    half = rot_dims // 2
+    if half > 0:
+        c, s = _rot_table(cos_sin, positions, half)
+        c, s = c[:, None, :], s[:, None, :]
+        for t_ in (q, k):
+            u, w_ = t_[..., :half].clone(), t_[..., half:2 * half].clone()
+            t_[..., :half] = u * c - w_ * s
+            t_[..., half:2 * half] = w_ * c + u * s
+    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * qscale.float()[None, :, None]
+    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
+    live = slots >= 0
+    sl = slots[live].long()
+    k_cache.view(-1, G, d)[sl] = k[live].to(k_cache.dtype)
+    v_cache.view(-1, G, dv)[sl] = v[live].to(v_cache.dtype)
+    return q.to(proj.dtype)
+
+
+def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate=None):
+    """Causal softmax attention of q [T, heads, dim] (already scaled) over paged keys / values;
+    query head h reads key/value head h // (heads / kv_heads); the output [T, heads * vdim] is
+    multiplied by sigmoid(gate) when a gate [T, heads * vdim] is given."""
+    T, H, d = q.shape
+    BSz, G, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    out = torch.zeros((T, H * dv), dtype=q.dtype, device=q.device)
+    qs, ql, cx = qstart.tolist(), qlen.tolist(), ctx.tolist()
+    for s in range(len(qs)):
+        n, c = ql[s], cx[s]
+        if n <= 0:
+            continue
+        nb = (c + BSz - 1) // BSz
+        blocks = block_tables[s, :nb].long()
+        K = k_cache[blocks].reshape(nb * BSz, G, d)[:c].float().repeat_interleave(H // G, 1)
+        V = v_cache[blocks].reshape(nb * BSz, G, dv)[:c].float().repeat_interleave(H // G, 1)
+        qq = q[qs[s]:qs[s] + n].float()
+        sc = torch.einsum("thd,uhd->htu", qq, K)
+        pos = torch.arange(c - n, c, device=q.device)
+        mask = torch.arange(c, device=q.device)[None, :] > pos[:, None]
+        sc = sc.masked_fill(mask[None], float("-inf"))
+        o = torch.einsum("htu,uhv->thv", torch.softmax(sc, -1), V).reshape(n, H * dv)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[qs[s]:qs[s] + n].float())
+        out[qs[s]:qs[s] + n] = o.to(q.dtype)
+    return out
+
+
+# ----------------------------------------------------------------------------- lightning attention, gated delta rule
+
+def lightning_attention(qkvg, heads, dim, vdim, decay, state, eps, norm_w, qstart, qlen, ctx, rows):
+    """Linear attention with a fixed decay per head over SiLU'd q, k, v: S <- decay S + k v^T,
+    o = S^T q; the heads of a token are RMS-normed together (weight ``norm_w``) and multiplied by
+    sigmoid(gate).  qkvg [T, >= 2 heads dim + 2 heads vdim] (q | k | v | gate); state
+    [slots, heads, dim, vdim] f32."""
+    T, H, d, dv = qkvg.shape[0], heads, dim, vdim
+    out = torch.zeros((T, H * dv), dtype=qkvg.dtype, device=qkvg.device)
+    dec = decay.float()
+    silu = torch.nn.functional.silu
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        blk = qkvg[q0:q0 + n].float()
+        q = silu(blk[:, :H * d]).reshape(n, H, d)
+        k = silu(blk[:, H * d:2 * H * d]).reshape(n, H, d)
+        v = silu(blk[:, 2 * H * d:2 * H * d + H * dv]).reshape(n, H, dv)
+        g = blk[:, 2 * H * d + H * dv:2 * H * d + 2 * H * dv]
+        S = state[row].clone() if cx - n > 0 else torch.zeros((H, d, dv), dtype=torch.float32, device=qkvg.device)
+        o = torch.empty((n, H, dv), dtype=torch.float32, device=qkvg.device)
+        for t in range(n):
+            S = dec[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[row] = S
+        o = rms_rows(o.reshape(n, H * dv), norm_w, eps, torch.float32)
+        out[q0:q0 + n] = (o * torch.sigmoid(g)).to(qkvg.dtype)
+    return out
+
+
+def conv_state_refill(x, conv_state, qstart, qlen, ctx, rows):
+    """conv_state[slot] <- the last K - 1 inputs of each sequence (x [T, >= C], state [slots, K - 1, C])."""
+    Km1, C = conv_state.shape[1], conv_state.shape[2]
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        hist = conv_state[row].float() if cx - n > 0 else torch.zeros((Km1, C), dtype=torch.float32, device=x.device)
+        u = torch.cat([hist, x[q0:q0 + n, :C].float()], 0)
+        conv_state[row] = u[u.shape[0] - Km1:].to(conv_state.dtype)
+
+
+def delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps, state, qstart, qlen, ctx, rows):
+    """Gated delta rule.  qkv [T, 2 kv_heads dim + heads vdim] (q | k | v, convolved and activated);
+    gba [T, >= heads vdim + 2 heads] (output gate | beta logits | decay logits).  Per head, with q
+    and k made unit vectors (sum of squares + 1e-6), q times dim^-1/2, beta = sigmoid(.),
+    g = exp(neg_a softplus(. + dt_bias)):  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;
+    o = S^T q.  Each head's o to unit RMS times ``norm_w`` times silu(gate).  state
+    [slots, heads, vdim, dim] f32 (transposed: a value column's state is contiguous)."""
+    T, H, G, d, dv = qkv.shape[0], heads, kv_heads, dim, vdim
+    out = torch.zeros((T, H * dv), dtype=qkv.dtype, device=qkv.device)
+    rep = H // G
+    for q0, n, cx, row in _seq_meta(qstart, qlen, ctx, rows):
+        blk = qkv[q0:q0 + n].float()
+        q = blk[:, :G * d].reshape(n, G, d)
+        k = blk[:, G * d:2 * G * d].reshape(n, G, d)
+        v = blk[:, 2 * G * d:2 * G * d + H * dv].reshape(n, H, dv)
+        q = q * torch.rsqrt(q.pow(2).sum(-1, keepdim=True) + 1e-6) * (d ** -0.5)
+        k = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+        q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
+        z = gba[q0:q0 + n].float()
+        gate, beta = z[:, :H * dv], torch.sigmoid(z[:, H * dv:H * dv + H])
+        g = torch.exp(neg_a.float()[None, :] * torch.nn.functional.softplus(z[:, H * dv + H:H * dv + 2 * H] + dt_bias.float()[None, :]))
+        S = state[row].clone() if cx - n > 0 else torch.zeros((H, dv, d), dtype=torch.float32, device=qkv.device)
+        o = torch.empty((n, H, dv), dtype=torch.float32, device=qkv.device)
+        for t in range(n):
+            S = g[t][:, None, None] * S
+            u = beta[t][:, None] * (v[t] - torch.einsum("hvd,hd->hv", S, k[t]))
+            S = S + u[:, :, None] * k[t][:, None, :]
+            o[t] = torch.einsum("hvd,hd->hv", S, q[t])
+        state[row] = S
+        o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()[None, None, :]
+        out[q0:q0 + n] = (o.reshape(n, H * dv) * torch.nn.functional.silu(gate)).to(qkv.dtype)
+    return out

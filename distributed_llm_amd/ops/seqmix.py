@@ -184,3 +184,122 @@ def dense_gate(ids, wts, E) -> torch.Tensor:
     g = torch.zeros((ids.shape[0], E), dtype=torch.float32, device=ids.device)   # fill kernel (graph-safe)
     ext.dense_gate(ids.to(torch.int32).contiguous(), wts.float().contiguous(), g)
     return g
+
+
+# ----------------------------------------------------------------------------- layers with a norm on both sides, depth average
+
+def resadd_norm(a: torch.Tensor, w_post: torch.Tensor, eps: float, x: torch.Tensor,
+                w_next: Optional[torch.Tensor] = None, x_next: Optional[torch.Tensor] = None,
+                b: Optional[torch.Tensor] = None, wa: Optional[torch.Tensor] = None,
+                wb: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The tail of a sublayer in one launch: ``x += rmsnorm(y) * w_post`` on the f32 stream, where y
+    is the sublayer's output ``a`` or, for two mixers side by side, ``(rmsnorm(a) wa + rmsnorm(b) wb) / 2``;
+    ``x_next`` (the model dtype) receives ``rmsnorm(x) * w_next``, the next sublayer's input."""
+    ext = _native(a)
+    if ext is None:
+        return ref.resadd_norm(a, w_post, eps, x, w_next, x_next, b, wa, wb)
+    ext.resadd_norm(a, b, wa, wb, w_post, float(eps), x, w_next, x_next)
+    return x
+
+
+def depth_mix(X: torch.Tensor, w: torch.Tensor, n: int, w_next: Optional[torch.Tensor] = None, eps: float = 0.0,
+              out_next: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Weighted sum over depth: ``X[n] = sum_{j<n} w[j] X[j]`` (X [slots, T, width] f32, w f32), plus
+    ``out_next = rmsnorm(X[n]) * w_next`` in the same launch."""
+    ext = _native(X)
+    if ext is None:
+        return ref.depth_mix(X, w, n, w_next, eps, out_next)
+    ext.depth_mix(X, w, int(n), w_next, float(eps), out_next)
+    return X[n]
+
+
+def gelu_erf(x: torch.Tensor) -> torch.Tensor:
+    """0.5 x (1 + erf(x / sqrt 2)) on bf16 or f32 activations."""
+    ext = _native(x)
+    if ext is None:
+        return ref.gelu_erf(x)
+    y = torch.empty_like(x)
+    ext.gelu_erf(x, y)
+    return y
+
+
+# ----------------------------------------------------------------------------- grouped-query attention over pages
+
+GQA_ROWS = 16      # (token, query head) rows per workgroup of the paged attention kernel
+
+
+def gqa_tokens_per_tile(heads: int, kv_heads: int) -> int:
+    """New tokens one attention workgroup covers (its rows are these tokens x the query heads of
+    one key/value head); the step's tile table (AttnMeta.latent_tiles) is built for this number."""
+    return max(1, GQA_ROWS // max(1, heads // kv_heads))
+
+
+def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots, k_cache,
+              v_cache) -> torch.Tensor:
+    """Rotate q and k (rotate-half, first ``rot_dims`` dims), bring every head to unit RMS, scale q
+    per head, write k and v to their page slots; returns q [T, heads, dim]."""
+    ext = _native(proj)
+    if ext is None:
+        return ref.attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots,
+                             k_cache, v_cache)
+    q = torch.zeros((proj.shape[0], heads, dim), dtype=proj.dtype, device=proj.device)
+    ext.attn_prep(proj, int(heads), int(kv_heads), int(dim), int(vdim), cos_sin, int(rot_dims), float(eps), qscale,
+                  positions, slots, k_cache, v_cache, q)
+    return q
+
+
+def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
+                        gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
+    softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
+    ``gqa_tokens_per_tile`` new tokens of a sequence."""
+    ext = _native(q)
+    if ext is None:
+        return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate)
+    out = torch.zeros((q.shape[0], q.shape[1] * v_cache.shape[3]), dtype=q.dtype, device=q.device)
+    ext.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0, gate, out)
+    return out
+
+
+# ----------------------------------------------------------------------------- lightning attention, gated delta rule
+
+def lightning_attention(qkvg, heads, dim, vdim, decay, state, eps, norm_w, qstart, qlen, ctx, rows,
+                        chunked: Optional[bool] = None) -> torch.Tensor:
+    """Decayed linear attention over SiLU'd q, k, v (no rotation, no key scale); a token's heads are
+    normed together and gated by a sigmoid.  Runs the retention kernels (token by token for decode
+    steps, chunked for prompt portions) in their raw-output form, then one norm-and-gate launch."""
+    ext = _native(qkvg)
+    if ext is None:
+        return ref.lightning_attention(qkvg, heads, dim, vdim, decay, state, eps, norm_w, qstart, qlen, ctx, rows)
+    T = qkvg.shape[0]
+    out = torch.zeros((T, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    if chunked is None:
+        chunked = T >= RETENTION_CHUNK_MIN * qstart.numel()
+    if not chunked and retention_step_lds(dim, vdim) > 150 * 1024:
+        chunked = True
+    raw = torch.zeros((T, heads, vdim), dtype=torch.float32, device=qkvg.device)
+    ext.lightning_attention(qkvg, int(heads), int(dim), int(vdim), decay, state, float(eps), norm_w, qstart, qlen, ctx,
+                            rows, out, raw, bool(chunked))
+    return out
+
+
+def conv_state_refill(x, conv_state, qstart, qlen, ctx, rows) -> None:
+    """Keep each sequence's last ``taps - 1`` convolution inputs in its slot."""
+    ext = _native(x)
+    if ext is None:
+        return ref.conv_state_refill(x, conv_state, qstart, qlen, ctx, rows)
+    ext.conv_state_refill(x, conv_state, qstart, qlen, ctx, rows)
+
+
+def delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps, state, qstart, qlen, ctx,
+               rows) -> torch.Tensor:
+    """Gated delta rule over convolved q | k | v with the gate, beta and decay logits in ``gba``;
+    unit q / k, decay, beta, the state [slots, heads, vdim, dim] and the per-head output norm in f32."""
+    ext = _native(qkv)
+    if ext is None:
+        return ref.delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps, state, qstart, qlen,
+                              ctx, rows)
+    out = torch.zeros((qkv.shape[0], heads * vdim), dtype=qkv.dtype, device=qkv.device)
+    ext.delta_rule(qkv, gba, int(heads), int(kv_heads), int(dim), int(vdim), neg_a, dt_bias, norm_w, float(eps), state,
+                   qstart, qlen, ctx, rows, out)
+    return out
