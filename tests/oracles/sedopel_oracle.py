@@ -146,3 +146,11 @@ def forward(cfg, weights, tokens, taps=None):
         if taps is not None:
             taps.append(x)
     return rms(x, eps, W["final.norm"]) @ W["head"].T
+
+
+def greedy(cfg, weights, prompt, n):
+    """n arg-max continuations of a prompt (the whole sequence is recomputed every step)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(torch.argmax(forward(cfg, weights, toks)[-1])))
+    return toks[len(prompt):]
