@@ -110,6 +110,8 @@ def parse():
                          "Llama-family model at equal size, prefill / decode throughput and mixer-kernel rooflines "
                          "(prints its own JSON object)")
     ap.add_argument("--arch-size", default="s", choices=["s", "m"])
+    ap.add_argument("--arch-design", default="filevik", choices=["filevik", "sedopel"],
+                    help="with --arch-bench: which layer-list design runs beside its closest Llama-family model")
     ap.add_argument("--arch-kernels-only", action="store_true")
     ap.add_argument("--trace", default=None,
                     help="write a Chrome trace (router/pool/engine spans, GPU decode time) to this path; "
@@ -487,7 +489,7 @@ def main() -> int:
     a = parse()
     if a.arch_bench:
         from distributed_llm_amd.bench import arch_bench
-        arch_bench.run(a.arch_size, kernels_only=a.arch_kernels_only)
+        arch_bench.run(a.arch_size, kernels_only=a.arch_kernels_only, design=a.arch_design)
         return 0
     if os.environ.get("DLLM_STACK_DUMP_S"):   # diagnostics: every thread's stack after S seconds (hang hunting)
         import faulthandler

@@ -1,8 +1,16 @@
-"""Layer-list (Filevik) models beside the closest Llama-family model at equal size: prefill and
-decode throughput through the engine, and the time of each mixer kernel against its roofline.
+"""Layer-list (Filevik, Sedopel) models beside the closest Llama-family model at equal size: prefill
+and decode throughput through the engine, and the time of each mixer kernel against its roofline.
 
-``python bench.py --arch-bench [--arch-size s|m]`` (random weights, synthetic tokens).  The default
-bench workload and its JSON contract are untouched; this prints one JSON object of its own.
+``python bench.py --arch-bench [--arch-design filevik|sedopel] [--arch-size s|m]`` (random weights,
+synthetic tokens).  The default bench workload and its JSON contract are untouched; this prints one
+JSON object of its own.
+
+The Sedopel stack alternates parallel layers (grouped-query softmax attention beside lightning
+attention, dense GELU feed-forward) and gated-delta-rule layers without a feed-forward; its
+comparison model is a dense Llama (grouped-query attention + SwiGLU of equal parameter count) of
+the same width and depth, and kernel by kernel: paged attention against the Llama attention kernels
+at the same head counts, lightning attention against retention, the delta rule against the
+selective scan.
 
 Sizes: width / layers of a small and a mid-size decoder.  The Filevik stack cycles mamba1 ->
 retention -> latent attention, each with routed squared-ReLU experts and a shared expert; the
@@ -29,6 +37,105 @@ SIZES = {
               lat_heads=16, lat_dim=128, lat_rot=64, lat_v=128, kv_rank=512, q_rank=1536, experts=8, top=2, ff=2048,
               shared=2048, vocab=32000),
 }
+
+
+SEDOPEL_SIZES = {
+    "s": dict(width=1024, layers=6, heads=16, kv_heads=4, dim=64, vdim=64, rot=32, l_heads=8, l_dim=64, l_vdim=128,
+              d_heads=8, d_kv_heads=4, d_dim=128, d_vdim=128, conv=4, ff=4096, vocab=32000),
+    "m": dict(width=2048, layers=12, heads=32, kv_heads=8, dim=64, vdim=64, rot=32, l_heads=16, l_dim=128, l_vdim=128,
+              d_heads=16, d_kv_heads=8, d_dim=128, d_vdim=128, conv=4, ff=8192, vocab=32000),
+}
+
+
+def sedopel_raw(z: dict) -> dict:
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"],
+                              "scale": z["dim"] ** -0.5 * 4.0, "rot": {"dims": z["rot"], "base": 10000.0}},
+                     "right": {"heads": z["l_heads"], "dim": z["l_dim"], "vdim": z["l_vdim"],
+                               "decay": [1.0 - 2.0 ** (-5 - i % 4) for i in range(z["l_heads"])]}},
+           "mlp": {"kind": "dense", "ff": z["ff"]}}
+    dlt = {"type": "delta", "mixer": {"heads": z["d_heads"], "kv_heads": z["d_kv_heads"], "dim": z["d_dim"],
+                                      "vdim": z["d_vdim"], "conv": z["conv"]}, "mlp": None}
+    return {"architecture": "Sedopel", "width": z["width"], "vocab": z["vocab"], "norm": {"eps": 1e-6},
+            "layers": [par if i % 2 == 0 else dlt for i in range(z["layers"])]}
+
+
+def dense_llama_twin(z: dict):
+    """Dense Llama of the same width, depth, vocabulary and attention heads, its SwiGLU width chosen
+    so that the parameter counts are equal."""
+    from ..models.configs import ModelConfig, sedopel_config
+    mk = lambda inter: ModelConfig(f"llama-{z['width']}", z["width"], z["layers"], z["heads"], z["kv_heads"], z["dim"],
+                                   inter, z["vocab"], 10000.0, 1e-6, 16384)
+    target = sedopel_config(sedopel_raw(z)).num_params()
+    inter = (target - mk(0).num_params()) // (3 * z["width"] * z["layers"])
+    return mk(max(64, inter // 64 * 64))
+
+
+def sedopel_kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 2048) -> Dict[str, dict]:
+    """Each Sedopel mixer kernel alone (bf16): prefill of one T-token sequence, decode of B sequences
+    at ``ctx``; time, the bound resource's minimum time, and their ratio."""
+    from .. import ops
+    from ..models.llama import AttnMeta
+    from ..ops import seqmix
+    dev, bf = "cuda", torch.bfloat16
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    res: Dict[str, dict] = {}
+
+    def rec(name, sec, bytes_, flops, peak_flops):
+        floor = max(bytes_ / PEAK_BW, flops / peak_flops)
+        res[name] = {"us": round(sec * 1e6, 1), "roofline_us": round(floor * 1e6, 2), "x_roofline": round(sec / floor, 1),
+                     "bound": "memory" if bytes_ / PEAK_BW >= flops / peak_flops else "compute"}
+
+    for tag, qlens, starts in (("prefill", [T], [0]), ("decode", [1] * B, [ctx] * B)):
+        n, S = sum(qlens), len(qlens)
+        qstart = i32([sum(qlens[:i]) for i in range(S)])
+        cxl = [a + b for a, b in zip(starts, qlens)]
+        qlen, cx, rows = i32(qlens), i32(cxl), i32(list(range(S)))
+        pos = i32([p for a, m in zip(starts, qlens) for p in range(a, a + m)])
+        keys = sum((a + (m + 1) / 2) * m for a, m in zip(starts, qlens))     # causal (query, key) pairs
+        # softmax attention over pages
+        H, G, d, dv = z["heads"], z["kv_heads"], z["dim"], z["vdim"]
+        nb = (max(cxl) + 15) // 16
+        bt = torch.arange(S * nb, dtype=torch.int32, device=dev).view(S, nb)
+        kc = (torch.randn(S * nb, 16, G, d, device=dev) * 0.3).to(bf)
+        vc = (torch.randn(S * nb, 16, G, dv, device=dev) * 0.3).to(bf)
+        proj = torch.randn(n, (H + G) * d + G * dv + H * dv, device=dev).to(bf)
+        table = ops.rope_cos_sin(ctx + T + 8, z["rot"], 10000.0, dev)
+        slots = i32([int(bt[i, p // 16]) * 16 + p % 16 for i, (a, m) in enumerate(zip(starts, qlens)) for p in range(a, a + m)])
+        qs = torch.full((H,), d ** -0.5, device=dev)
+        q = seqmix.attn_prep(proj, H, G, d, dv, table, z["rot"], 1e-6, qs, pos, slots, kc, vc)
+        rec(f"attn_prep_{tag}", _timed(lambda: seqmix.attn_prep(proj, H, G, d, dv, table, z["rot"], 1e-6, qs, pos, slots, kc, vc)),
+            n * ((H + G) * d + G * dv) * 4 + n * H * d * 2, n * (H + G) * d * 8, PEAK_F32)
+        meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=cx, tile_seq=None, tile_tok0=None,
+                        last_idx=None, host_qlen=qlens)
+        ts, tt = meta.latent_tiles(1, dev, seqmix.gqa_tokens_per_tile(H, G))
+        gate = proj[:, (H + G) * d + G * dv:]
+        rec(f"attention_{tag}",
+            _timed(lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, gate), 3),
+            sum(cxl) * G * (d + dv) * 2 + n * H * (d + 2 * dv) * 2, keys * H * 2 * (d + dv), PEAK_BF16)
+        # lightning attention
+        Hl, dl, dvl = z["l_heads"], z["l_dim"], z["l_vdim"]
+        qkvg = torch.randn(n, 2 * Hl * dl + 2 * Hl * dvl, device=dev).to(bf)
+        dec, st = torch.full((Hl,), 0.98, device=dev), torch.zeros(S, Hl, dl, dvl, device=dev)
+        nw = torch.ones(Hl * dvl, device=dev)
+        rec(f"lightning_{tag}",
+            _timed(lambda: seqmix.lightning_attention(qkvg, Hl, dl, dvl, dec, st, 1e-6, nw, qstart, qlen, cx, rows)),
+            n * (2 * Hl * dl + 3 * Hl * dvl) * 2 + (S * Hl * dl * dvl * 8 if tag == "decode" else 0),
+            n * Hl * dl * dvl * 4 if tag == "decode" else n * Hl * (4 * dl * dvl + 2 * 64 * (dl + dvl)), PEAK_F32)
+        # gated delta rule (+ its convolution)
+        Hd, Gd, dd, dvd, K = z["d_heads"], z["d_kv_heads"], z["d_dim"], z["d_vdim"], z["conv"]
+        C = 2 * Gd * dd + Hd * dvd
+        pr = torch.randn(n, C + Hd * dvd + 2 * Hd, device=dev).to(bf)
+        conv_s, sd = torch.zeros(S, K - 1, C, device=dev, dtype=bf), torch.zeros(S, Hd, dvd, dd, device=dev)
+        w, b_ = torch.randn(C, K, device=dev) * 0.5, torch.zeros(C, device=dev)
+        qkv = seqmix.causal_conv_silu(pr, w, b_, conv_s, qstart, qlen, cx, rows)
+        na, dtb, hn = -torch.rand(Hd, device=dev), torch.zeros(Hd, device=dev), torch.ones(dvd, device=dev)
+        rec(f"delta_conv_{tag}", _timed(lambda: seqmix.causal_conv_silu(pr, w, b_, conv_s, qstart, qlen, cx, rows)),
+            n * C * 4 + (S * (K - 1) * C * 2 if tag == "decode" else 0), n * C * 2 * K, PEAK_F32)
+        rec(f"delta_rule_{tag}",
+            _timed(lambda: seqmix.delta_rule(qkv, pr[:, C:], Hd, Gd, dd, dvd, na, dtb, hn, 1e-6, sd, qstart, qlen, cx, rows)),
+            n * (C + 2 * Hd * dvd) * 2 + (S * Hd * dd * dvd * 8 if tag == "decode" else 0), n * Hd * dd * dvd * 6, PEAK_F32)
+    return res
 
 
 def filevik_raw(z: dict) -> dict:
@@ -196,8 +303,21 @@ def llama_kernel_rooflines(T: int = 4096, B: int = 64, ctx: int = 2048, nq: int 
     return res
 
 
-def run(size: str = "s", kernels_only: bool = False) -> dict:
-    from ..models.configs import filevik_config
+def run(size: str = "s", kernels_only: bool = False, design: str = "filevik") -> dict:
+    from ..models.configs import filevik_config, sedopel_config
+    if design == "sedopel":
+        z = SEDOPEL_SIZES[size]
+        out = {"bench": "arch", "design": design, "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}
+        out["sedopel_kernels"] = sedopel_kernel_rooflines(z)
+        out["filevik_kernels"] = kernel_rooflines(SIZES[size])
+        out["llama_kernels"] = llama_kernel_rooflines(nq=z["heads"], nkv=z["kv_heads"], d=z["dim"])
+        if not kernels_only:
+            prompts, batches = [512, 2048], [1, 16, 64]
+            out["sedopel"] = engine_throughput(sedopel_config(sedopel_raw(z), name=f"sedopel-{size}"), prompts, batches,
+                                               ctx=1024, new=32, rows=64)
+            out["llama"] = engine_throughput(dense_llama_twin(z), prompts, batches, ctx=1024, new=32, rows=64)
+        print(json.dumps(out))
+        return out
     z = SIZES[size]
     out = {"bench": "arch", "size": size, "dtype": "bf16", "data": "synthetic", "sizes": z}
     out["filevik_kernels"] = kernel_rooflines(z)
