@@ -73,10 +73,11 @@ int dllm_conv_refill(const void*, long, int, void*, int, int, const int*, const 
 int dllm_delta_rule(const void*, long, const void*, long, int, int, int, int, int, const float*, const float*, const float*,
                     float, float*, const int*, const int*, const int*, const int*, float*, void*, int, long, hipStream_t);
 int dllm_attn_prep(const void*, long, int, int, int, int, int, const float*, int, int, float, const float*, const int*,
-                   const int*, void*, void*, void*, long, hipStream_t);
-int dllm_gqa_tile_tokens(int, int);
+                   const int*, void*, void*, void*, long, int, hipStream_t);
+int dllm_gqa_tile_tokens(int, int, int);
+int dllm_gqa_mfma_ok(int, int, int, int, int, int);
 int dllm_paged_gqa(const void*, const void*, const void*, int, const int*, int, int, const int*, const int*, const int*,
-                   const int*, const int*, int, const void*, long, void*, int, int, int, int, hipStream_t);
+                   const int*, const int*, int, const void*, long, void*, int, int, int, int, int, hipStream_t);
 int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
 int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
 int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
@@ -1617,29 +1618,31 @@ void attn_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, 
   TORCH_CHECK(qscale.numel() == H && pos.numel() == T && slots.numel() == T, "qscale / positions / slots lengths");
   for (auto* c : {&kc, &vc})
     TORCH_CHECK(c->is_cuda() && c->scalar_type() == proj.scalar_type() && c->is_contiguous() && c->dim() == 4 &&
-                    c->size(2) == G,
-                "paged cache [blocks, block, G, width] in the activations' dtype");
-  TORCH_CHECK(kc.size(3) == d && vc.size(3) == dv && kc.size(0) == vc.size(0) && kc.size(1) == vc.size(1), "cache widths");
+                    c->size(1) == G,
+                "paged caches K [blocks, G, block, d], V [blocks, G, dv, block] in the activations' dtype");
+  TORCH_CHECK(kc.size(3) == d && vc.size(2) == dv && kc.size(0) == vc.size(0) && kc.size(2) == vc.size(3), "cache widths");
   TORCH_CHECK(q.is_cuda() && q.scalar_type() == proj.scalar_type() && q.is_contiguous() && q.numel() == T * H * d, "q [T, H, d]");
   ok(dllm_attn_prep(proj.data_ptr(), proj.stride(0), f, (int)H, (int)G, (int)d, (int)dv, cos_sin.data_ptr<float>(),
                     (int)cos_sin.size(1), (int)rot, (float)eps, qscale.data_ptr<float>(), pos.data_ptr<int>(),
-                    slots.data_ptr<int>(), kc.data_ptr(), vc.data_ptr(), q.data_ptr(), (long)T, stream()),
+                    slots.data_ptr<int>(), kc.data_ptr(), vc.data_ptr(), q.data_ptr(), (long)T, (int)kc.size(2), stream()),
      "attn_prep");
 }
 
 void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, torch::Tensor bt, torch::Tensor qstart,
                          torch::Tensor qlen, torch::Tensor ctx, torch::Tensor tile_seq, torch::Tensor tile_tok0,
-                         c10::optional<torch::Tensor> gate, torch::Tensor out) {
+                         c10::optional<torch::Tensor> gate, torch::Tensor out, bool mfma) {
   const bool f = act_f32(q, "q");
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous(), "q [T, H, d]");
   const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
   for (auto* c : {&kc, &vc})
     TORCH_CHECK(c->is_cuda() && c->scalar_type() == q.scalar_type() && c->is_contiguous() && c->dim() == 4,
-                "paged cache [blocks, block, G, width] in the dtype of q");
-  const int64_t G = kc.size(2), dv = vc.size(3);
-  TORCH_CHECK(G >= 1 && H % G == 0 && kc.size(3) == d && vc.size(2) == G && kc.size(0) == vc.size(0) &&
-                  kc.size(1) == vc.size(1) && dv <= 256,
+                "paged caches K [blocks, G, block, d], V [blocks, G, dv, block] in the dtype of q");
+  const int64_t G = kc.size(1), dv = vc.size(2);
+  TORCH_CHECK(G >= 1 && H % G == 0 && kc.size(3) == d && vc.size(1) == G && kc.size(0) == vc.size(0) &&
+                  kc.size(2) == vc.size(3) && dv <= 256,
               "cache shapes; vdim <= 256");
+  TORCH_CHECK(!mfma || dllm_gqa_mfma_ok(f, (int)H, (int)G, (int)d, (int)dv, (int)kc.size(2)),
+              "shape outside the matrix-core kernel's range");
   check_i32(bt, "block_tables");
   TORCH_CHECK(bt.dim() == 2 && bt.stride(1) == 1, "block_tables [S, blocks]");
   for (auto* t : {&qstart, &qlen, &ctx, &tile_seq, &tile_tok0}) check_i32(*t, "sequence / tile metadata");
@@ -1659,9 +1662,9 @@ void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, to
                   out.size(0) == T && out.size(1) == H * dv,
               "out [T, H dv]");
   const int rc = dllm_paged_gqa(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), f, bt.data_ptr<int>(), (int)bt.stride(0),
-                                (int)kc.size(1), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
+                                (int)kc.size(2), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                                 tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), gp, ldg,
-                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, stream());
+                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, (int)mfma, stream());
   TORCH_CHECK(rc != -2, "head widths do not fit the LDS");
   ok(rc, "paged_gqa_attention");
 }
@@ -1781,7 +1784,11 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("delta_rule", &delta_rule);
   m.def("attn_prep", &attn_prep);
   m.def("paged_gqa_attention", &paged_gqa_attention);
-  m.def("gqa_tile_tokens", [](int64_t H, int64_t G) { return (int64_t)dllm_gqa_tile_tokens((int)H, (int)G); });
+  m.def("gqa_tile_tokens",
+        [](int64_t H, int64_t G, bool mfma) { return (int64_t)dllm_gqa_tile_tokens((int)H, (int)G, (int)mfma); });
+  m.def("gqa_mfma_ok", [](bool f32, int64_t H, int64_t G, int64_t d, int64_t dv, int64_t bs) {
+    return (bool)dllm_gqa_mfma_ok((int)f32, (int)H, (int)G, (int)d, (int)dv, (int)bs);
+  });
   m.def("latent_kv_write", &latent_kv_write);
   m.def("latent_attention", &latent_attention, py::arg("qa"), py::arg("q"), py::arg("dim"), py::arg("rot"),
         py::arg("positions"), py::arg("cos_sin"), py::arg("cache"), py::arg("block_tables"), py::arg("qstart"),

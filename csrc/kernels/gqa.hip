@@ -9,8 +9,17 @@
 //               four rows), f32 online softmax per row, then a lane owns value dims for the weighted
 //               sum (one V read feeds four rows).  The output is multiplied by sigmoid(gate).
 //
-// Cache layout: K [blocks, block, G, d], V [blocks, block, G, dv] (bf16 or f32 like the activations);
-// every score, weight and sum is f32.
+//   paged_gqa_mfma  the bf16 form on the matrix cores: 64 rows per workgroup, 16 per wave, so a row's
+//               softmax never leaves its wave.  Q stays in registers as MFMA operands; a 64-key tile is
+//               staged once for the four waves (K row-major, V already transposed in its page);
+//               scores on v_mfma_f32_16x16x32_bf16 with f32 sums; online softmax in the accumulator
+//               layout (row maxima over the 16 lanes of a DPP row); the weights go through the wave's
+//               own LDS patch as bf16 hi + lo parts, so the weighted sum sees them to 16 bits of
+//               mantissa through two MFMAs.  Key blocks above a wave's newest row are skipped.
+//
+// Cache layout: K [blocks, G, block, d], V [blocks, G, dv, block] (bf16 or f32 like the activations;
+// V is kept transposed inside its page because the weighted sum contracts over keys); every score,
+// weight and sum is f32.
 #include "common.h"
 
 namespace {
@@ -27,17 +36,19 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const T* __restrict__ pr
                                                         const float* __restrict__ cos_sin, int tab_w, int rot, float eps,
                                                         const float* __restrict__ qscale, const int* __restrict__ pos,
                                                         const int* __restrict__ slots, T* __restrict__ kc,
-                                                        T* __restrict__ vc, T* __restrict__ q) {
+                                                        T* __restrict__ vc, T* __restrict__ q, int BSZ) {
   const long tok = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const T* r = proj + tok * ld;
   const int slot = slots[tok];
+  const long blk = slot >= 0 ? slot / BSZ : 0;
+  const int off = slot >= 0 ? slot % BSZ : 0;
   const int half = rot >> 1;
   const float* cs = cos_sin + (long)pos[tok] * tab_w;
-  for (int hh = wave; hh < H + G; hh += 4) {
+  const int hh = blockIdx.y * 4 + wave;     // q heads, then k heads, are consecutive in the projection
+  if (hh < H + G && (hh < H || slot >= 0)) {
     const bool is_q = hh < H;
-    if (!is_q && slot < 0) continue;
-    const T* x = r + (long)hh * d;    // q heads, then k heads, are consecutive in the projection
+    const T* x = r + (long)hh * d;
     float ss = 0.f;
     for (int i = lane; i < d; i += 64) {
       float v = ldf(x + i);
@@ -51,7 +62,7 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const T* __restrict__ pr
     }
     ss = wave_sum(ss);
     const float sc = (is_q ? qscale[hh] : 1.f) / sqrtf(ss / (float)d + eps);
-    T* dst = is_q ? q + (tok * H + hh) * d : kc + ((long)slot * G + (hh - H)) * d;
+    T* dst = is_q ? q + (tok * H + hh) * d : kc + ((blk * G + (hh - H)) * BSZ + off) * d;
     for (int i = lane; i < d; i += 64) {
       float v = ldf(x + i);
       if (i < rot) {
@@ -63,9 +74,10 @@ __global__ void __launch_bounds__(256) attn_prep_kernel(const T* __restrict__ pr
       stf(dst + i, v * sc);
     }
   }
-  if (slot >= 0) {
+  if (slot >= 0) {   // values: this workgroup's share of the G * dv entries
     const T* v = r + (long)(H + G) * d;
-    for (int i = threadIdx.x; i < G * dv; i += 256) vc[(long)slot * G * dv + i] = v[i];
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < G * dv; i += gridDim.y * 256)
+      vc[((blk * G + i / dv) * dv + i % dv) * BSZ + off] = v[i];
   }
 }
 
@@ -123,7 +135,7 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
       float v = 0.f;
       if (kk < nk) {
         const int pk = k0 + kk;
-        v = ldf(kc + (((long)btr[pk / BSZ] * BSZ + pk % BSZ) * G + g) * d + i);
+        v = ldf(kc + (((long)btr[pk / BSZ] * G + g) * BSZ + pk % BSZ) * d + i);
       }
       Ks[kk * dp + i] = v;
     }
@@ -132,7 +144,7 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
       float v = 0.f;
       if (kk < nk) {
         const int pk = k0 + kk;
-        v = ldf(vc + (((long)btr[pk / BSZ] * BSZ + pk % BSZ) * G + g) * dv + jx);
+        v = ldf(vc + (((long)btr[pk / BSZ] * G + g) * dv + jx) * BSZ + pk % BSZ);
       }
       Vs[e] = v;
     }
@@ -197,6 +209,184 @@ __global__ void __launch_bounds__(256) paged_gqa_kernel(const T* __restrict__ q,
   }
 }
 
+// ---------------------------------------------------------------- bf16 on the matrix cores
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false)));
+  return v;
+}
+__device__ __forceinline__ float row16_add(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+
+constexpr int GM_ROWS = 64, GM_KT = 64, GM_BS = 16;   // rows per workgroup, keys per tile, keys per page
+
+// SZ >= max(d, dv) in {64, 128, 256}: d is walked in SZ / 32 MFMA steps, dv in SZ / 16 column blocks
+// (steps and blocks past the real widths are skipped).  d % 8 == 0 (16-byte key rows).
+// MFMA operand layout (16x16x32): with lr = lane & 15, g4 = lane >> 4, A holds row lr, contraction
+// indices 8 g4 .. 8 g4 + 7; B holds column lr, the same indices; the accumulator holds rows
+// 4 g4 .. 4 g4 + 3 of column lr.
+template <int SZ>
+__global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restrict__ q, const u16* __restrict__ kc,
+                                                             const u16* __restrict__ vc, const int* __restrict__ bt,
+                                                             int bt_ld, const int* __restrict__ qstart,
+                                                             const int* __restrict__ qlen, const int* __restrict__ ctx,
+                                                             const int* __restrict__ tile_seq,
+                                                             const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
+                                                             long ldg, u16* __restrict__ out, int H, int G, int d, int dv,
+                                                             int TQ) {
+  constexpr int DS = SZ / 32, VB = SZ / 16, NKB = GM_KT / 16;
+  constexpr int KSTR = SZ + 8, VSTR = GM_KT + 8, PSTR = GM_KT + 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
+  const int s = tile_seq[blockIdx.x];
+  const int n = qlen[s];
+  const int tok0 = tile_tok0[blockIdx.x];
+  if (n <= 0 || tok0 >= n) return;   // the whole workgroup (padding tiles)
+  const int g = blockIdx.y, R = H / G;
+  const int nq = min(TQ, n - tok0), nrows = nq * R;
+  const int q0 = qstart[s], p0 = ctx[s] - n;
+  u16* ksh = reinterpret_cast<u16*>(smraw);          // [KT][KSTR]
+  u16* vtr = ksh + GM_KT * KSTR;                      // [SZ][VSTR]: values transposed, [dim][key]
+  u16* pw = vtr + SZ * VSTR;                          // [4 waves][hi | lo][16][PSTR]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, g4 = lane >> 4;
+  u16* phi = pw + wave * (2 * 16 * PSTR);
+  u16* plo = phi + 16 * PSTR;
+  // row rr -> (token tok0 + rr / R, query head g R + rr % R)
+  bf16x8 qa[DS];
+  {
+    const int row = 16 * wave + lr;
+    const bool rk = row < nrows;
+    const u16* qp = q + ((long)(q0 + tok0 + (rk ? row / R : 0)) * H + g * R + (rk ? row % R : 0)) * d;
+#pragma unroll
+    for (int st = 0; st < DS; ++st) {
+      const int c = st * 32 + 8 * g4;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (rk && c < d) v = *reinterpret_cast<const uint4*>(qp + c);
+      qa[st] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  int rpos[4];
+  float m[4], l[4];
+  f32x4 acc[VB];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = 16 * wave + 4 * g4 + i;
+    rpos[i] = row < nrows ? p0 + tok0 + row / R : -1;     // -1: sees no key
+    m[i] = -INFINITY;
+    l[i] = 0.f;
+  }
+#pragma unroll
+  for (int cb = 0; cb < VB; ++cb) acc[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int wave_last = 16 * wave < nrows ? p0 + tok0 + (min(16 * wave + 15, nrows - 1)) / R : -1;
+  const int last = p0 + tok0 + nq - 1;   // the newest key any row sees
+  const int* btr = bt + (long)s * bt_ld;
+  const int kchunks = SZ / 8;            // 16-byte chunks of a staged key row
+  for (int k0 = 0; k0 <= last; k0 += GM_KT) {
+    const int nk = min(GM_KT, last + 1 - k0);
+    __syncthreads();   // the previous tile is consumed
+    for (int e = tid; e < GM_KT * kchunks; e += 256) {
+      const int kk = e / kchunks, c = (e % kchunks) * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (kk < nk && c < d) {
+        const int pk = k0 + kk;
+        v = *reinterpret_cast<const uint4*>(kc + (((long)btr[pk >> 4] * G + g) * GM_BS + (pk & 15)) * d + c);
+      }
+      *reinterpret_cast<uint4*>(ksh + kk * KSTR + c) = v;
+    }
+    // values: a page holds [dv][16 keys]; entry (dim j, page pg, half hf) is 8 keys = 16 bytes
+    for (int e = tid; e < SZ * (GM_KT / 8); e += 256) {
+      const int j = e / (GM_KT / 8), c = e % (GM_KT / 8), pg = c >> 1, hf = c & 1;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (j < dv && 16 * pg < nk)
+        v = *reinterpret_cast<const uint4*>(vc + (((long)btr[(k0 >> 4) + pg] * G + g) * dv + j) * GM_BS + 8 * hf);
+      *reinterpret_cast<uint4*>(vtr + j * VSTR + 8 * c) = v;
+    }
+    __syncthreads();
+    if (k0 > wave_last) continue;   // this wave's rows see nothing of the tile (the barriers above are uniform)
+    f32x4 sacc[NKB];
+#pragma unroll
+    for (int kb = 0; kb < NKB; ++kb) {
+      sacc[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (k0 + 16 * kb > wave_last) continue;
+      const u16* bp = ksh + (16 * kb + lr) * KSTR + 8 * g4;
+#pragma unroll
+      for (int st = 0; st < DS; ++st) {
+        if (st * 32 < d) {
+          const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + st * 32));
+          sacc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[st], b, sacc[kb], 0, 0, 0);
+        }
+      }
+    }
+    float alpha[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        const bool vis = k0 + 16 * kb + lr <= rpos[i];
+        mx = fmaxf(mx, vis ? sacc[kb][i] : -INFINITY);
+      }
+      mx = row16_max(mx);
+      const float mn = fmaxf(m[i], mx);
+      alpha[i] = mn > -INFINITY ? expf(m[i] - mn) : 1.f;   // m = -inf before the first visible key: 0, and acc, l are 0
+      m[i] = mn;
+      l[i] *= alpha[i];
+#pragma unroll
+      for (int kb = 0; kb < NKB; ++kb) {
+        const bool vis = k0 + 16 * kb + lr <= rpos[i];
+        const float p = (vis && mn > -INFINITY) ? expf(sacc[kb][i] - mn) : 0.f;
+        l[i] += p;
+        const u16 hi = f2bf(p);
+        phi[(4 * g4 + i) * PSTR + 16 * kb + lr] = hi;
+        plo[(4 * g4 + i) * PSTR + 16 * kb + lr] = f2bf(p - bf2f(hi));
+      }
+    }
+    __builtin_amdgcn_wave_barrier();   // the patch is this wave's own: its LDS writes are in order before the reads
+#pragma unroll
+    for (int cb = 0; cb < VB; ++cb) {
+      if (cb * 16 >= dv) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[cb][i] *= alpha[i];
+      const u16* bp = vtr + (16 * cb + lr) * VSTR + 8 * g4;
+#pragma unroll
+      for (int ks = 0; ks < GM_KT; ks += 32) {
+        if (k0 + ks > wave_last) continue;
+        const bf16x8 bv = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp + ks));
+        const bf16x8 ah = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(phi + lr * PSTR + ks + 8 * g4));
+        const bf16x8 al = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(plo + lr * PSTR + ks + 8 * g4));
+        acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bv, acc[cb], 0, 0, 0);
+        acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al, bv, acc[cb], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lt = row16_add(l[i]);
+    const int row = 16 * wave + 4 * g4 + i;
+    if (row >= nrows) continue;
+    const long tok = q0 + tok0 + row / R;
+    const int h = g * R + row % R;
+    const float inv = 1.f / lt;
+#pragma unroll
+    for (int cb = 0; cb < VB; ++cb) {
+      const int jx = 16 * cb + lr;
+      if (jx >= dv) continue;
+      float o = acc[cb][i] * inv;
+      if (gate) o *= 1.f / (1.f + expf(-bf2f(gate[tok * ldg + (long)h * dv + jx])));
+      out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
+    }
+  }
+}
+
+long gqa_mfma_lds(int SZ) { return 2L * (GM_KT * (SZ + 8) + (long)SZ * (GM_KT + 8) + 4L * 2 * 16 * (GM_KT + 8)); }
+
 long gqa_lds(int d, int dv, int KT) { return 4L * (GA_ROWS * d + (long)KT * (d | 1) + (long)KT * dv + GA_ROWS * 64); }
 
 #define ENSURE_LDS(kernel, bytes)                                                                          \
@@ -233,30 +423,53 @@ int launch_gqa_t(int nj, dim3 grid, long lds, hipStream_t st, const void* q, con
 
 extern "C" int dllm_attn_prep(const void* proj, long ld, int f32, int H, int G, int d, int dv, const float* cos_sin,
                               int tab_w, int rot, float eps, const float* qscale, const int* pos, const int* slots, void* kc,
-                              void* vc, void* q, long T, hipStream_t st) {
+                              void* vc, void* q, long T, int BSZ, hipStream_t st) {
   if (T <= 0) return 0;
   if (rot < 0 || rot > d || (rot & 1) || rot > tab_w) return -1;
+  const dim3 grid((unsigned)T, (H + G + 3) / 4);
   if (f32)
-    hipLaunchKernelGGL(attn_prep_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, (const float*)proj, ld, H, G, d, dv, cos_sin,
-                       tab_w, rot, eps, qscale, pos, slots, (float*)kc, (float*)vc, (float*)q);
+    hipLaunchKernelGGL(attn_prep_kernel<float>, grid, dim3(256), 0, st, (const float*)proj, ld, H, G, d, dv, cos_sin, tab_w, rot,
+                       eps, qscale, pos, slots, (float*)kc, (float*)vc, (float*)q, BSZ);
   else
-    hipLaunchKernelGGL(attn_prep_kernel<u16>, dim3((unsigned)T), dim3(256), 0, st, (const u16*)proj, ld, H, G, d, dv, cos_sin,
-                       tab_w, rot, eps, qscale, pos, slots, (u16*)kc, (u16*)vc, (u16*)q);
+    hipLaunchKernelGGL(attn_prep_kernel<u16>, grid, dim3(256), 0, st, (const u16*)proj, ld, H, G, d, dv, cos_sin, tab_w, rot, eps,
+                       qscale, pos, slots, (u16*)kc, (u16*)vc, (u16*)q, BSZ);
   return (int)hipGetLastError();
 }
 
+// The matrix-core form takes bf16, 16-key pages, key rows of whole 16-byte vectors, widths <= 256 and
+// at most 64 query heads per key/value head.
+extern "C" int dllm_gqa_mfma_ok(int f32, int H, int G, int d, int dv, int BSZ) {
+  return !f32 && BSZ == GM_BS && G >= 1 && H % G == 0 && H / G <= GM_ROWS && d % 8 == 0 && d <= 256 && dv <= 256 && d >= 8;
+}
+
 // tokens one workgroup covers for H / G query heads per key/value head
-extern "C" int dllm_gqa_tile_tokens(int H, int G) {
-  const int R = H / G;
-  return R >= GA_ROWS ? 1 : GA_ROWS / R;
+extern "C" int dllm_gqa_tile_tokens(int H, int G, int mfma) {
+  const int R = H / G, rows = mfma ? GM_ROWS : GA_ROWS;
+  return R >= rows ? 1 : rows / R;
 }
 
 extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int f32, const int* bt, int bt_ld, int BSZ,
                               const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
-                              int n_tiles, const void* gate, long ldg, void* out, int H, int G, int d, int dv,
+                              int n_tiles, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int mfma,
                               hipStream_t st) {
   if (n_tiles <= 0) return 0;
   if (G < 1 || H % G || dv > 256 || d < 1) return -1;
+  if (mfma) {
+    if (!dllm_gqa_mfma_ok(f32, H, G, d, dv, BSZ)) return -1;
+    const int sz = d > dv ? d : dv;
+    const dim3 grid(n_tiles, G);
+    const int TQ = dllm_gqa_tile_tokens(H, G, 1);
+#define GQM(SZ)                                                                                                          \
+  do {                                                                                                                   \
+    const long lds = gqa_mfma_lds(SZ);                                                                                   \
+    ENSURE_LDS(paged_gqa_mfma_kernel<SZ>, lds);                                                                          \
+    hipLaunchKernelGGL(paged_gqa_mfma_kernel<SZ>, grid, dim3(256), lds, st, (const u16*)q, (const u16*)kc, (const u16*)vc, bt, \
+                       bt_ld, qstart, qlen, ctx, tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, d, dv, TQ); \
+  } while (0)
+    if (sz <= 64) GQM(64); else if (sz <= 128) GQM(128); else GQM(256);
+#undef GQM
+    return (int)hipGetLastError();
+  }
   int KT = 64;
   if (gqa_lds(d, dv, KT) > 150 * 1024) KT = 32;
   const long lds = gqa_lds(d, dv, KT);
@@ -264,7 +477,7 @@ extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int
   const int R = H / G;
   const dim3 grid(n_tiles, G, (R + GA_ROWS - 1) / GA_ROWS);
   const int nj = (dv + 63) / 64;
-  const int TQ = dllm_gqa_tile_tokens(H, G);
+  const int TQ = dllm_gqa_tile_tokens(H, G, 0);
   if (f32)
     return launch_gqa_t<float>(nj, grid, lds, st, q, kc, vc, bt, bt_ld, BSZ, qstart, qlen, ctx, tile_seq, tile_tok0, gate, ldg,
                                out, H, G, d, dv, TQ, KT);

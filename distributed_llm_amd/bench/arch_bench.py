@@ -97,8 +97,8 @@ def sedopel_kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 204
         H, G, d, dv = z["heads"], z["kv_heads"], z["dim"], z["vdim"]
         nb = (max(cxl) + 15) // 16
         bt = torch.arange(S * nb, dtype=torch.int32, device=dev).view(S, nb)
-        kc = (torch.randn(S * nb, 16, G, d, device=dev) * 0.3).to(bf)
-        vc = (torch.randn(S * nb, 16, G, dv, device=dev) * 0.3).to(bf)
+        kc = (torch.randn(S * nb, G, 16, d, device=dev) * 0.3).to(bf)
+        vc = (torch.randn(S * nb, G, dv, 16, device=dev) * 0.3).to(bf)
         proj = torch.randn(n, (H + G) * d + G * dv + H * dv, device=dev).to(bf)
         table = ops.rope_cos_sin(ctx + T + 8, z["rot"], 10000.0, dev)
         slots = i32([int(bt[i, p // 16]) * 16 + p % 16 for i, (a, m) in enumerate(zip(starts, qlens)) for p in range(a, a + m)])
@@ -108,10 +108,11 @@ def sedopel_kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 204
             n * ((H + G) * d + G * dv) * 4 + n * H * d * 2, n * (H + G) * d * 8, PEAK_F32)
         meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=cx, tile_seq=None, tile_tok0=None,
                         last_idx=None, host_qlen=qlens)
-        ts, tt = meta.latent_tiles(1, dev, seqmix.gqa_tokens_per_tile(H, G))
+        mfma = seqmix.gqa_use_mfma(q, H, G, d, dv, 16)
+        ts, tt = meta.latent_tiles(1, dev, seqmix.gqa_tokens_per_tile(H, G, mfma))
         gate = proj[:, (H + G) * d + G * dv:]
         rec(f"attention_{tag}",
-            _timed(lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, gate), 3),
+            _timed(lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, gate, mfma), 3),
             sum(cxl) * G * (d + dv) * 2 + n * H * (d + 2 * dv) * 2, keys * H * 2 * (d + dv), PEAK_BF16)
         # lightning attention
         Hl, dl, dvl = z["l_heads"], z["l_dim"], z["l_vdim"]

@@ -297,7 +297,8 @@ class HybridModel:
         sequences: (conv inputs [slots, taps - 1, inner], scan state [slots, inner, state] f32) /
         (retention state [slots, heads, dim, vdim] f32,) / delta: (conv inputs [slots, taps - 1,
         q | k | v channels], state [slots, heads, vdim, dim] f32) / parallel: (paged keys [blocks,
-        block, kv_heads, dim], paged values [.., vdim], lightning state [slots, heads, dim, vdim] f32)."""
+        kv_heads, block, dim], paged values [blocks, kv_heads, vdim, block], lightning state [slots,
+        heads, dim, vdim] f32)."""
         dev, out = self.device, []
         for L in self.cfg.layers:
             m = L.mixer
@@ -307,8 +308,8 @@ class HybridModel:
                             torch.zeros((slots, m.heads, m.vdim, m.dim), dtype=torch.float32, device=dev)))
             elif m.kind == "parallel":
                 a, b = m.left, m.right
-                out.append((torch.zeros((num_blocks, block_size, a.kv_heads, a.dim), dtype=self.dtype, device=dev),
-                            torch.zeros((num_blocks, block_size, a.kv_heads, a.vdim), dtype=self.dtype, device=dev),
+                out.append((torch.zeros((num_blocks, a.kv_heads, block_size, a.dim), dtype=self.dtype, device=dev),
+                            torch.zeros((num_blocks, a.kv_heads, a.vdim, block_size), dtype=self.dtype, device=dev),
                             torch.zeros((slots, b.heads, b.dim, b.vdim), dtype=torch.float32, device=dev)))
             elif m.kind == "mamba1":
                 out.append((torch.zeros((slots, max(m.conv - 1, 0), m.inner), dtype=self.dtype, device=dev),
@@ -388,10 +389,11 @@ class HybridModel:
         table = self._table(a) if rot else self._any_table()
         q = seqmix.attn_prep(proj, a.heads, a.kv_heads, a.dim, a.vdim, table, rot, eps, L["qscale"], positions,
                              meta.slots, k_cache, v_cache)
-        ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(a.heads, a.kv_heads))
+        mfma = seqmix.gqa_use_mfma(q, a.heads, a.kv_heads, a.dim, a.vdim, k_cache.shape[2])
+        ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(a.heads, a.kv_heads, mfma))
         gate = proj[:, nl - a.heads * a.vdim:nl]
         lo = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
-                                        gate)
+                                        gate, mfma)
         ro = seqmix.lightning_attention(proj[:, nl:], b.heads, b.dim, b.vdim, L["decay"], state, eps, L["rnorm"],
                                         meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
         return _mm(lo, L["lo"]), _mm(ro, L["ro"])

@@ -583,8 +583,8 @@ def gelu_erf(x):
 def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots, k_cache, v_cache):
     """proj [T, >= heads dim + kv_heads (dim + vdim)] (q | k | v).  q and k: rotate-half positions on
     the first ``rot_dims`` dims of each head, then each head to unit RMS; q times ``qscale[head]``.
-    k and v go to their page slots (k_cache [blocks, block, kv_heads, dim], v_cache [..., vdim]);
-    returns q [T, heads, dim]."""
+    k and v go to their page slots (k_cache [blocks, kv_heads, block, dim], v_cache [blocks,
+    kv_heads, vdim, block]: values transposed inside a page); returns q [T, heads, dim]."""
     T, H, G, d, dv = proj.shape[0], heads, kv_heads, dim, vdim
     pf = proj.float()
     q = pf[:, :H * d].reshape(T, H, d).clone()
@@ -602,8 +602,9 @@ def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, 
     k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps)
     live = slots >= 0
     sl = slots[live].long()
-    k_cache.view(-1, G, d)[sl] = k[live].to(k_cache.dtype)
-    v_cache.view(-1, G, dv)[sl] = v[live].to(v_cache.dtype)
+    BSz = k_cache.shape[2]
+    k_cache[sl // BSz, :, sl % BSz] = k[live].to(k_cache.dtype)
+    v_cache[sl // BSz, :, :, sl % BSz] = v[live].to(v_cache.dtype)
     return q.to(proj.dtype)
 
 
@@ -612,7 +613,7 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ga
     query head h reads key/value head h // (heads / kv_heads); the output [T, heads * vdim] is
     multiplied by sigmoid(gate) when a gate [T, heads * vdim] is given."""
     T, H, d = q.shape
-    BSz, G, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    G, BSz, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     out = torch.zeros((T, H * dv), dtype=q.dtype, device=q.device)
     qs, ql, cx = qstart.tolist(), qlen.tolist(), ctx.tolist()
     for s in range(len(qs)):
@@ -621,8 +622,8 @@ def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, ga
             continue
         nb = (c + BSz - 1) // BSz
         blocks = block_tables[s, :nb].long()
-        K = k_cache[blocks].reshape(nb * BSz, G, d)[:c].float().repeat_interleave(H // G, 1)
-        V = v_cache[blocks].reshape(nb * BSz, G, dv)[:c].float().repeat_interleave(H // G, 1)
+        K = k_cache[blocks].transpose(1, 2).reshape(nb * BSz, G, d)[:c].float().repeat_interleave(H // G, 1)
+        V = v_cache[blocks].permute(0, 3, 1, 2).reshape(nb * BSz, G, dv)[:c].float().repeat_interleave(H // G, 1)
         qq = q[qs[s]:qs[s] + n].float()
         sc = torch.einsum("thd,uhd->htu", qq, K)
         pos = torch.arange(c - n, c, device=q.device)

@@ -225,19 +225,30 @@ def gelu_erf(x: torch.Tensor) -> torch.Tensor:
 
 # ----------------------------------------------------------------------------- grouped-query attention over pages
 
-GQA_ROWS = 16      # (token, query head) rows per workgroup of the paged attention kernel
+GQA_ROWS = 16          # (token, query head) rows per workgroup of the vector-ALU paged attention kernel
+GQA_ROWS_MFMA = 64     # ... of the matrix-core kernel (bf16)
 
 
-def gqa_tokens_per_tile(heads: int, kv_heads: int) -> int:
+def gqa_use_mfma(q_like: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int, block: int) -> bool:
+    """The matrix-core attention kernel runs bf16 models on the GPU whose shapes it takes
+    (``DLLM_GQA_MFMA=0`` keeps the vector-ALU kernel that f32 models run)."""
+    if not q_like.is_cuda or q_like.dtype != torch.bfloat16 or os.environ.get("DLLM_GQA_MFMA", "1") != "1":
+        return False
+    ext = _native(q_like)
+    return ext is not None and bool(ext.gqa_mfma_ok(False, int(heads), int(kv_heads), int(dim), int(vdim), int(block)))
+
+
+def gqa_tokens_per_tile(heads: int, kv_heads: int, mfma: bool = False) -> int:
     """New tokens one attention workgroup covers (its rows are these tokens x the query heads of
     one key/value head); the step's tile table (AttnMeta.latent_tiles) is built for this number."""
-    return max(1, GQA_ROWS // max(1, heads // kv_heads))
+    return max(1, (GQA_ROWS_MFMA if mfma else GQA_ROWS) // max(1, heads // kv_heads))
 
 
 def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots, k_cache,
               v_cache) -> torch.Tensor:
     """Rotate q and k (rotate-half, first ``rot_dims`` dims), bring every head to unit RMS, scale q
-    per head, write k and v to their page slots; returns q [T, heads, dim]."""
+    per head, write k and v to their page slots (k_cache [blocks, kv_heads, block, dim], v_cache
+    [blocks, kv_heads, vdim, block]); returns q [T, heads, dim]."""
     ext = _native(proj)
     if ext is None:
         return ref.attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots,
@@ -249,15 +260,16 @@ def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, 
 
 
 def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
-                        gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        gate: Optional[torch.Tensor] = None, mfma: bool = False) -> torch.Tensor:
     """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
     softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
-    ``gqa_tokens_per_tile`` new tokens of a sequence."""
+    ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence."""
     ext = _native(q)
     if ext is None:
         return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate)
-    out = torch.zeros((q.shape[0], q.shape[1] * v_cache.shape[3]), dtype=q.dtype, device=q.device)
-    ext.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0, gate, out)
+    out = torch.zeros((q.shape[0], q.shape[1] * v_cache.shape[2]), dtype=q.dtype, device=q.device)
+    ext.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0, gate, out,
+                            bool(mfma))
     return out
 
 

@@ -178,3 +178,145 @@ def test_moe_relu2_grouped(T):
     assert seqmix.moe_ffn_relu2_ok(x, w1)
     y = seqmix.moe_ffn_relu2(x, ids, w, w1, w2)
     torch.testing.assert_close(y.float(), ref.moe_ffn_relu2(x, ids, w, w1, w2).float(), atol=3e-2, rtol=3e-2)
+
+
+# ----------------------------------------------------------------------------- pre/post-norm tails, depth average, GELU
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("n", [24, 200, 1032])
+@pytest.mark.parametrize("pair", [False, True])
+def test_resadd_norm(dt, n, pair):
+    torch.manual_seed(2)
+    a = torch.randn(9, n + 5, device=DEV).to(dt)[:, 2:2 + n]
+    b = torch.randn(9, n, device=DEV).to(dt) if pair else None
+    wa, wb, wp, wn = (torch.randn(n, device=DEV) for _ in range(4))
+    for w_next in (wn, None):
+        x1 = torch.randn(9, n, device=DEV)
+        x2 = x1.clone()
+        h1, h2 = torch.empty(9, n, device=DEV, dtype=dt), torch.empty(9, n, device=DEV, dtype=dt)
+        kw = dict(b=b, wa=wa, wb=wb) if pair else {}
+        seqmix.resadd_norm(a, wp, 1e-5, x1, w_next, h1, **kw)
+        ref.resadd_norm(a, wp, 1e-5, x2, w_next, h2, **kw)
+        torch.testing.assert_close(x1, x2, atol=2e-5, rtol=2e-5)
+        torch.testing.assert_close(h1.float(), h2.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_depth_mix_and_gelu(dt):
+    torch.manual_seed(3)
+    X1 = torch.randn(6, 11, 72, device=DEV)
+    X2 = X1.clone()
+    w, wn = torch.randn(5, device=DEV), torch.randn(72, device=DEV)
+    h1, h2 = torch.empty(11, 72, device=DEV, dtype=dt), torch.empty(11, 72, device=DEV, dtype=dt)
+    for n in (1, 3, 5):
+        seqmix.depth_mix(X1, w, n, wn, 1e-5, h1)
+        ref.depth_mix(X2, w, n, wn, 1e-5, h2)
+        torch.testing.assert_close(X1, X2, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(h1.float(), h2.float(), **tol(dt))
+    x = (torch.randn(7, 100, device=DEV) * 3).to(dt)
+    torch.testing.assert_close(seqmix.gelu_erf(x).float(), ref.gelu_erf(x).float(), **tol(dt))
+
+
+# ----------------------------------------------------------------------------- grouped-query attention over pages
+
+def _pages(case, G, d, dv, dt, BSz=16):
+    qlens, starts = case
+    T, qstart, qlen, ctx, rows, pos = batch(qlens, starts)
+    nb = max((a + n + BSz - 1) // BSz for a, n in zip(starts, qlens))
+    S = len(qlens)
+    perm = torch.randperm(S * nb + 3, device=DEV)[:S * nb].to(torch.int32).view(S, nb)     # pages out of order
+    kc = (torch.randn(S * nb + 3, G, BSz, d, device=DEV) * 0.5).to(dt)
+    vc = torch.randn(S * nb + 3, G, dv, BSz, device=DEV).to(dt)
+    slots = i32([int(perm[i, p // BSz]) * BSz + p % BSz for i, (a, n) in enumerate(zip(starts, qlens)) for p in range(a, a + n)])
+    return T, qstart, qlen, ctx, pos, perm.contiguous(), kc, vc, slots
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES + [([40, 3], [90, 130])])
+@pytest.mark.parametrize("H,G,d,dv,rot", [(4, 2, 16, 8, 8), (6, 3, 96, 48, 24), (3, 3, 40, 72, 40), (34, 2, 8, 5, 0),
+                                          (8, 1, 64, 64, 32), (2, 1, 136, 200, 64)])
+def test_attn_prep_and_paged_gqa(dt, case, H, G, d, dv, rot):
+    from distributed_llm_amd.models.llama import AttnMeta
+    torch.manual_seed(4)
+    T, qstart, qlen, ctx, pos, bt, kc, vc, slots = _pages(case, G, d, dv, dt)
+    proj = torch.randn(T, (H + G) * d + G * dv + H * dv + 3, device=DEV).to(dt)
+    table = ops.rope_cos_sin(256, max(rot, 2), 100.0, DEV)
+    qscale = torch.rand(H, device=DEV) * 2 + 0.5
+    kc2, vc2 = kc.clone(), vc.clone()
+    q1 = seqmix.attn_prep(proj, H, G, d, dv, table, rot, 1e-5, qscale, pos, slots, kc, vc)
+    q2 = ref.attn_prep(proj, H, G, d, dv, table, rot, 1e-5, qscale, pos, slots, kc2, vc2)
+    torch.testing.assert_close(q1.float(), q2.float(), **tol(dt))
+    torch.testing.assert_close(kc.float(), kc2.float(), **tol(dt))
+    torch.testing.assert_close(vc.float(), vc2.float(), atol=0, rtol=0)
+    gate = proj[:, (H + G) * d + G * dv:(H + G) * d + G * dv + H * dv]
+    want = ref.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, gate).float()
+    meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
+                    last_idx=None, host_qlen=case[0])
+    forms = [False] + ([True] if seqmix.gqa_use_mfma(q2, H, G, d, dv, 16) else [])
+    for mfma in forms:
+        ts, tt = meta.latent_tiles(1, DEV, seqmix.gqa_tokens_per_tile(H, G, mfma))
+        got = seqmix.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, ts, tt, gate, mfma).float()
+        torch.testing.assert_close(got, want, **tol(dt))
+
+
+def test_paged_gqa_mfma_keeps_small_weights():
+    """One key carries almost all of a row's weight; the others' weights are ~1e-3 and their values
+    large: the hi + lo split of the weights keeps their sum (a bf16-only weight would lose ~0.4 %)."""
+    from distributed_llm_amd.models.llama import AttnMeta
+    torch.manual_seed(5)
+    H, G, d, dv, n = 2, 1, 64, 64, 200
+    dt = torch.bfloat16
+    T, qstart, qlen, ctx, pos, bt, kc, vc, slots = _pages(([n], [0]), G, d, dv, dt)
+    q = (torch.randn(n, H, d, device=DEV) * 0.6).to(dt)
+    vc = (vc.float() * 50).to(dt)
+    want = ref.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, ctx).float()
+    meta = AttnMeta(slots=None, block_tables=bt, qstart=qstart, qlen=qlen, ctx=ctx, tile_seq=None, tile_tok0=None,
+                    last_idx=None, host_qlen=[n])
+    ts, tt = meta.latent_tiles(1, DEV, seqmix.gqa_tokens_per_tile(H, G, True))
+    got = seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, ctx, ts, tt, None, True).float()
+    assert float((got - want).abs().max()) < 0.02 * float(want.abs().max())
+    torch.testing.assert_close(got, want, atol=0.35, rtol=8e-3)      # outputs rounded to bf16 at |o| ~ 50
+
+
+# ----------------------------------------------------------------------------- lightning attention, gated delta rule
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("H,d,dv", [(2, 8, 6), (4, 64, 32), (1, 40, 130), (3, 128, 128)])
+@pytest.mark.parametrize("chunked", [False, True])
+def test_lightning_attention(dt, case, H, d, dv, chunked):
+    torch.manual_seed(6)
+    T, qstart, qlen, ctx, rows, pos = batch(*case)
+    qkvg = torch.randn(T, 2 * H * d + 2 * H * dv + 5, device=DEV).to(dt)
+    decay = torch.tensor([0.6, 0.9, 0.99, 1.0][:H], device=DEV)
+    st1 = torch.randn(len(case[0]), H, d, dv, device=DEV) * 0.3
+    st2 = st1.clone()
+    nw = torch.randn(H * dv, device=DEV)
+    got = seqmix.lightning_attention(qkvg, H, d, dv, decay, st1, 1e-5, nw, qstart, qlen, ctx, rows, chunked=chunked)
+    want = ref.lightning_attention(qkvg, H, d, dv, decay, st2, 1e-5, nw, qstart, qlen, ctx, rows)
+    torch.testing.assert_close(got.float(), want.float(), **tol(dt))
+    torch.testing.assert_close(st1, st2, atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("H,G,d,dv,K", [(4, 2, 8, 6, 3), (6, 3, 64, 32, 4), (1, 1, 20, 33, 1), (2, 1, 200, 18, 2), (2, 2, 128, 128, 4)])
+def test_delta_rule_and_conv_refill(dt, case, H, G, d, dv, K):
+    torch.manual_seed(7)
+    T, qstart, qlen, ctx, rows, pos = batch(*case)
+    C = 2 * G * d + H * dv
+    S = len(case[0])
+    proj = torch.randn(T, C + H * dv + 2 * H, device=DEV).to(dt)
+    qkv = torch.nn.functional.silu(torch.randn(T, C, device=DEV)).to(dt)
+    neg_a, dtb, nw = -torch.rand(H, device=DEV) * 2, torch.randn(H, device=DEV), torch.randn(dv, device=DEV)
+    st1 = torch.randn(S, H, dv, d, device=DEV) * 0.3
+    st2 = st1.clone()
+    got = seqmix.delta_rule(qkv, proj[:, C:], H, G, d, dv, neg_a, dtb, nw, 1e-5, st1, qstart, qlen, ctx, rows)
+    want = ref.delta_rule(qkv, proj[:, C:], H, G, d, dv, neg_a, dtb, nw, 1e-5, st2, qstart, qlen, ctx, rows)
+    torch.testing.assert_close(got.float(), want.float(), **tol(dt))
+    torch.testing.assert_close(st1, st2, atol=1e-4, rtol=1e-4)
+    c1 = torch.randn(S, K - 1, C, device=DEV).to(dt)
+    c2 = c1.clone()
+    seqmix.conv_state_refill(proj, c1, qstart, qlen, ctx, rows)
+    ref.conv_state_refill(proj, c2, qstart, qlen, ctx, rows)
+    torch.testing.assert_close(c1.float(), c2.float(), atol=0, rtol=0)
