@@ -287,34 +287,47 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
   const int wave_last = 16 * wave < nrows ? p0 + tok0 + (min(16 * wave + 15, nrows - 1)) / R : -1;
   const int last = p0 + tok0 + nq - 1;   // the newest key any row sees
   const int* btr = bt + (long)s * bt_ld;
-  const int kchunks = SZ / 8;            // 16-byte chunks of a staged key row
-  for (int k0 = 0; k0 <= last; k0 += GM_KT) {
+  constexpr int KCH = SZ / 8;            // 16-byte chunks of a staged key row
+  constexpr int NF = SZ / 32;            // chunks of K, and of V, a thread moves per tile
+  // Score block kb, column lr stands for key 4 lr + kb of the tile (K rows are staged in that order),
+  // so a lane's four blocks are four neighbouring keys and its weights leave as 8-byte vectors.
+  uint4 pk_[NF], pv_[NF];
+  auto fetch = [&](int k0) {
     const int nk = min(GM_KT, last + 1 - k0);
-    __syncthreads();   // the previous tile is consumed
-    for (int e = tid; e < GM_KT * kchunks; e += 256) {
-      const int kk = e / kchunks, c = (e % kchunks) * 8;
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      const int e = tid + 256 * f;
+      const int kk = e / KCH, c = (e % KCH) * 8;
+      pk_[f] = make_uint4(0u, 0u, 0u, 0u);
       if (kk < nk && c < d) {
         const int pk = k0 + kk;
-        v = *reinterpret_cast<const uint4*>(kc + (((long)btr[pk >> 4] * G + g) * GM_BS + (pk & 15)) * d + c);
+        pk_[f] = *reinterpret_cast<const uint4*>(kc + (((long)btr[pk >> 4] * G + g) * GM_BS + (pk & 15)) * d + c);
       }
-      *reinterpret_cast<uint4*>(ksh + kk * KSTR + c) = v;
-    }
-    // values: a page holds [dv][16 keys]; entry (dim j, page pg, half hf) is 8 keys = 16 bytes
-    for (int e = tid; e < SZ * (GM_KT / 8); e += 256) {
-      const int j = e / (GM_KT / 8), c = e % (GM_KT / 8), pg = c >> 1, hf = c & 1;
-      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      // values: a page holds [dv][16 keys]; entry (dim j, page pg, half hf) is 8 keys = 16 bytes
+      const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8), pg = cc >> 1, hf = cc & 1;
+      pv_[f] = make_uint4(0u, 0u, 0u, 0u);
       if (j < dv && 16 * pg < nk)
-        v = *reinterpret_cast<const uint4*>(vc + (((long)btr[(k0 >> 4) + pg] * G + g) * dv + j) * GM_BS + 8 * hf);
-      *reinterpret_cast<uint4*>(vtr + j * VSTR + 8 * c) = v;
+        pv_[f] = *reinterpret_cast<const uint4*>(vc + (((long)btr[(k0 >> 4) + pg] * G + g) * dv + j) * GM_BS + 8 * hf);
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 <= last; k0 += GM_KT) {
+    __syncthreads();   // the previous tile is consumed
+#pragma unroll
+    for (int f = 0; f < NF; ++f) {
+      const int e = tid + 256 * f;
+      const int kk = e / KCH, c = (e % KCH) * 8;
+      *reinterpret_cast<uint4*>(ksh + (16 * (kk & 3) + (kk >> 2)) * KSTR + c) = pk_[f];
+      const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8);
+      *reinterpret_cast<uint4*>(vtr + j * VSTR + 8 * cc) = pv_[f];
+    }
+    if (k0 + GM_KT <= last) fetch(k0 + GM_KT);   // the next tile's loads fly under this tile's products
     __syncthreads();
     if (k0 > wave_last) continue;   // this wave's rows see nothing of the tile (the barriers above are uniform)
     f32x4 sacc[NKB];
 #pragma unroll
     for (int kb = 0; kb < NKB; ++kb) {
       sacc[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (k0 + 16 * kb > wave_last) continue;
       const u16* bp = ksh + (16 * kb + lr) * KSTR + 8 * g4;
 #pragma unroll
       for (int st = 0; st < DS; ++st) {
@@ -325,28 +338,32 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
       }
     }
     float alpha[4];
+    const int key0 = k0 + 4 * lr;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float mx = -INFINITY;
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) {
-        const bool vis = k0 + 16 * kb + lr <= rpos[i];
-        mx = fmaxf(mx, vis ? sacc[kb][i] : -INFINITY);
-      }
+      for (int kb = 0; kb < NKB; ++kb) mx = fmaxf(mx, key0 + kb <= rpos[i] ? sacc[kb][i] : -INFINITY);
       mx = row16_max(mx);
       const float mn = fmaxf(m[i], mx);
-      alpha[i] = mn > -INFINITY ? expf(m[i] - mn) : 1.f;   // m = -inf before the first visible key: 0, and acc, l are 0
+      const bool any = mn > -INFINITY;
+      alpha[i] = any ? __expf(m[i] - mn) : 1.f;   // m = -inf before the first visible key: 0, and acc, l are 0
       m[i] = mn;
       l[i] *= alpha[i];
+      uint32_t hi[NKB], lo[NKB];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        const bool vis = k0 + 16 * kb + lr <= rpos[i];
-        const float p = (vis && mn > -INFINITY) ? expf(sacc[kb][i] - mn) : 0.f;
+        const float p = (any && key0 + kb <= rpos[i]) ? __expf(sacc[kb][i] - mn) : 0.f;
         l[i] += p;
-        const u16 hi = f2bf(p);
-        phi[(4 * g4 + i) * PSTR + 16 * kb + lr] = hi;
-        plo[(4 * g4 + i) * PSTR + 16 * kb + lr] = f2bf(p - bf2f(hi));
+        // p is in [0, 1]: round to nearest even without the special cases
+        uint32_t u = __float_as_uint(p);
+        u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+        hi[kb] = u;
+        uint32_t w = __float_as_uint(p - __uint_as_float(u << 16));
+        lo[kb] = (w + 0x7fffu + ((w >> 16) & 1u)) >> 16;
       }
+      *reinterpret_cast<uint2*>(phi + (4 * g4 + i) * PSTR + 4 * lr) = make_uint2(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16));
+      *reinterpret_cast<uint2*>(plo + (4 * g4 + i) * PSTR + 4 * lr) = make_uint2(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16));
     }
     __builtin_amdgcn_wave_barrier();   // the patch is this wave's own: its LDS writes are in order before the reads
 #pragma unroll
