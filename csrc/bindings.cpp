@@ -77,7 +77,7 @@ int dllm_attn_prep(const void*, long, int, int, int, int, int, const float*, int
 int dllm_gqa_tile_tokens(int, int, int);
 int dllm_gqa_mfma_ok(int, int, int, int, int, int);
 int dllm_paged_gqa(const void*, const void*, const void*, int, const int*, int, int, const int*, const int*, const int*,
-                   const int*, const int*, int, const void*, long, void*, int, int, int, int, int, hipStream_t);
+                   const int*, const int*, int, const void*, long, void*, int, int, int, int, int, int, float*, hipStream_t);
 int dllm_relu2_scale(const void*, int, const float*, int, int, void*, long, int, hipStream_t);
 int dllm_dense_gate(const int*, const float*, float*, long, int, int, hipStream_t);
 int dllm_latent_kv_write(const void*, long, int, int, int, const float*, float, const int*, const float*, int, const int*,
@@ -1594,7 +1594,8 @@ void delta_rule(torch::Tensor qkv, torch::Tensor gba, int64_t H, int64_t G, int6
                   out.size(0) == T && out.size(1) == H * dv,
               "out [T, H dv]");
   auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
-  auto raw = torch::zeros({T, H, dv}, torch::TensorOptions().dtype(torch::kFloat32).device(qkv.device()));
+  // f32 outputs before the per-head norm: written and read for tokens of live sequences only
+  auto raw = torch::empty({T, H, dv}, torch::TensorOptions().dtype(torch::kFloat32).device(qkv.device()));
   ok(dllm_delta_rule(qkv.data_ptr(), qkv.stride(0), gba.data_ptr(), gba.stride(0), f, (int)H, (int)G, (int)d, (int)dv,
                      neg_a.data_ptr<float>(), dt_bias.data_ptr<float>(), norm_w.data_ptr<float>(), (float)eps,
                      state.data_ptr<float>(), m.qstart, m.qlen, m.ctx, m.rows, raw.data_ptr<float>(), out.data_ptr(), m.S,
@@ -1630,7 +1631,8 @@ void attn_prep(torch::Tensor proj, int64_t H, int64_t G, int64_t d, int64_t dv, 
 
 void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, torch::Tensor bt, torch::Tensor qstart,
                          torch::Tensor qlen, torch::Tensor ctx, torch::Tensor tile_seq, torch::Tensor tile_tok0,
-                         c10::optional<torch::Tensor> gate, torch::Tensor out, bool mfma) {
+                         c10::optional<torch::Tensor> gate, torch::Tensor out, bool mfma, int64_t splits,
+                         c10::optional<torch::Tensor> part) {
   const bool f = act_f32(q, "q");
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous(), "q [T, H, d]");
   const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
@@ -1661,10 +1663,18 @@ void paged_gqa_attention(torch::Tensor q, torch::Tensor kc, torch::Tensor vc, to
   TORCH_CHECK(out.is_cuda() && out.scalar_type() == q.scalar_type() && out.is_contiguous() && out.dim() == 2 &&
                   out.size(0) == T && out.size(1) == H * dv,
               "out [T, H dv]");
+  float* pptr = nullptr;
+  TORCH_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || mfma), "key splits: 1..64, matrix-core kernel only");
+  if (splits > 1) {
+    TORCH_CHECK(part.has_value(), "key splits need a workspace");
+    check_f32(*part, "split workspace");
+    TORCH_CHECK(part->numel() >= (int64_t)tile_seq.numel() * G * splits * 64 * (dv + 2), "split workspace size");
+    pptr = part->data_ptr<float>();
+  }
   const int rc = dllm_paged_gqa(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), f, bt.data_ptr<int>(), (int)bt.stride(0),
                                 (int)kc.size(2), qstart.data_ptr<int>(), qlen.data_ptr<int>(), ctx.data_ptr<int>(),
                                 tile_seq.data_ptr<int>(), tile_tok0.data_ptr<int>(), (int)tile_seq.numel(), gp, ldg,
-                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, (int)mfma, stream());
+                                out.data_ptr(), (int)H, (int)G, (int)d, (int)dv, (int)mfma, (int)splits, pptr, stream());
   TORCH_CHECK(rc != -2, "head widths do not fit the LDS");
   ok(rc, "paged_gqa_attention");
 }
@@ -1783,7 +1793,10 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("conv_state_refill", &conv_state_refill);
   m.def("delta_rule", &delta_rule);
   m.def("attn_prep", &attn_prep);
-  m.def("paged_gqa_attention", &paged_gqa_attention);
+  m.def("paged_gqa_attention", &paged_gqa_attention, py::arg("q"), py::arg("k_cache"), py::arg("v_cache"),
+        py::arg("block_tables"), py::arg("qstart"), py::arg("qlen"), py::arg("ctx"), py::arg("tile_seq"),
+        py::arg("tile_tok0"), py::arg("gate"), py::arg("out"), py::arg("mfma"), py::arg("splits") = 1,
+        py::arg("part") = py::none());
   m.def("gqa_tile_tokens",
         [](int64_t H, int64_t G, bool mfma) { return (int64_t)dllm_gqa_tile_tokens((int)H, (int)G, (int)mfma); });
   m.def("gqa_mfma_ok", [](bool f32, int64_t H, int64_t G, int64_t d, int64_t dv, int64_t bs) {

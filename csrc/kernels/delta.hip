@@ -8,9 +8,10 @@
 //     u_j = beta (v_j - g a);   o_j = g b + u_j (k . q);   S_j <- g S_j + k u_j
 // so the kernel gives a column to 16 lanes (a DPP row: the two dot products are row rotations), a
 // workgroup 16 columns of one (sequence, head), and walks the tokens in order.  Tokens are staged in
-// groups of 16: raw q / k rows in LDS, unit norms and k . q by one wave per token, beta and the decay
+// groups of 16: raw q / k rows in LDS, unit norms and k . q by one DPP row per token, beta and the decay
 // (sigmoid, softplus, two exponentials) by one lane per token, so the serial part of a token is two
-// multiply-add sweeps over the lane's state registers and the row sums.  All of it is f32; the
+// multiply-add sweeps over the lane's state registers and the row sums.  A group's inputs are fetched
+// into registers while the previous group's recurrence runs.  All of it is f32; the
 // state [slots, heads, vdim, dim] keeps a column contiguous.  delta_finish norms each head's output
 // (unit RMS times a weight shared by the heads) and applies the SiLU gate.
 #include "common.h"
@@ -50,7 +51,7 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(const T* __restrict__ q
   const int h = blockIdx.y, s = blockIdx.z;
   const int n = qlen[s];
   if (n <= 0) return;   // the whole workgroup
-  const int tid = threadIdx.x, sub = tid & 15, col = tid >> 4, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, sub = tid & 15, col = tid >> 4;
   const int j0 = blockIdx.x * DR_COLS, j = j0 + col;
   const bool live = j < dv;
   const int kvh = h / (H / G);
@@ -65,62 +66,89 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(const T* __restrict__ q
   const long oq = (long)kvh * d, ok = (long)G * d + (long)kvh * d, ov = 2L * G * d + (long)h * dv;
   const long ob = (long)H * dv + h, oa = (long)H * dv + H + h;
   const float na = neg_a[h], dtb = dt_bias[h], qscale = 1.f / sqrtf((float)d);
+  // a group's inputs are fetched into registers one group ahead, so their latency hides under the
+  // previous group's recurrence: NS entries of q and of k, one of v, and (lanes < 16) the two logits
+  float pq[NS], pk[NS], pv = 0.f, pb = 0.f, pa = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = min(DR_TT, n - t0);
+#pragma unroll
+    for (int r = 0; r < NS; ++r) {
+      const int e = tid + 256 * r;
+      const int tt = e / DP, c = e % DP;       // c = r' * 16 + sub'  ->  dim sub' * NS + r'
+      const int i = (c & 15) * NS + (c >> 4);
+      const bool okx = tt < nt && i < d;
+      const T* row = qkv + (long)(q0 + t0 + (okx ? tt : 0)) * ldq;
+      pq[r] = okx ? ldf(row + oq + i) : 0.f;
+      pk[r] = okx ? ldf(row + ok + i) : 0.f;
+    }
+    {
+      const int tt = tid / DR_COLS, c = tid % DR_COLS;
+      pv = (tt < nt && j0 + c < dv) ? ldf(qkv + (long)(q0 + t0 + tt) * ldq + ov + j0 + c) : 0.f;
+    }
+    if (tid < nt) {
+      const T* row = gba + (long)(q0 + t0 + tid) * ldg;
+      pb = ldf(row + ob);
+      pa = ldf(row + oa);
+    }
+  };
+  fetch(0);
   for (int t0 = 0; t0 < n; t0 += DR_TT) {
     const int nt = min(DR_TT, n - t0);
     __syncthreads();   // the previous group is consumed
-    for (int e = tid; e < nt * DP; e += 256) {
-      const int tt = e / DP, c = e % DP;       // c = r * 16 + sub'  ->  dim sub' * NS + r
-      const int i = (c & 15) * NS + (c >> 4);
-      const T* r = qkv + (long)(q0 + t0 + tt) * ldq;
-      qs[e] = i < d ? ldf(r + oq + i) : 0.f;
-      ks[e] = i < d ? ldf(r + ok + i) : 0.f;
+#pragma unroll
+    for (int r = 0; r < NS; ++r) {
+      qs[tid + 256 * r] = pq[r];
+      ks[tid + 256 * r] = pk[r];
     }
-    for (int e = tid; e < nt * DR_COLS; e += 256) {
-      const int tt = e / DR_COLS, c = e % DR_COLS;
-      vs[e] = j0 + c < dv ? ldf(qkv + (long)(q0 + t0 + tt) * ldq + ov + j0 + c) : 0.f;
-    }
+    vs[tid] = pv;
     if (tid < nt) {
-      const T* r = gba + (long)(q0 + t0 + tid) * ldg;
-      const float z = ldf(r + oa) + dtb;
+      const float z = pa + dtb;
       const float sp_ = z > 20.f ? z : log1pf(expf(z));
-      bg[tid * 4] = 1.f / (1.f + expf(-ldf(r + ob)));
+      bg[tid * 4] = 1.f / (1.f + expf(-pb));
       bg[tid * 4 + 1] = expf(na * sp_);
     }
     __syncthreads();
-    for (int tt = wave; tt < nt; tt += 4) {   // unit q (times dim^-1/2) and k, and k . q
-      float sq = 0.f, sk = 0.f;
-      for (int c = lane; c < DP; c += 64) {
-        const float qv = qs[tt * DP + c], kv = ks[tt * DP + c];
-        sq += qv * qv;
-        sk += kv * kv;
+    if (t0 + DR_TT < n) fetch(t0 + DR_TT);
+    {   // unit q (times dim^-1/2) and k, and k . q: the 16 lanes of a DPP row take one token
+      const int tt = tid >> 4;
+      float qv[NS], kv[NS], sq = 0.f, sk = 0.f;
+#pragma unroll
+      for (int r = 0; r < NS; ++r) {
+        qv[r] = qs[tt * DP + r * 16 + sub];
+        kv[r] = ks[tt * DP + r * 16 + sub];
+        sq += qv[r] * qv[r];
+        sk += kv[r] * kv[r];
       }
-      sq = wave_sum(sq);
-      sk = wave_sum(sk);
+      sq = row16_sum(sq);
+      sk = row16_sum(sk);
       const float rq = qscale / sqrtf(sq + 1e-6f), rk = 1.f / sqrtf(sk + 1e-6f);
       float kq = 0.f;
-      for (int c = lane; c < DP; c += 64) {
-        const float qv = qs[tt * DP + c] * rq, kv = ks[tt * DP + c] * rk;
-        qs[tt * DP + c] = qv;
-        ks[tt * DP + c] = kv;
-        kq += qv * kv;
+#pragma unroll
+      for (int r = 0; r < NS; ++r) {
+        qv[r] *= rq;
+        kv[r] *= rk;
+        qs[tt * DP + r * 16 + sub] = qv[r];
+        ks[tt * DP + r * 16 + sub] = kv[r];
+        kq += qv[r] * kv[r];
       }
-      kq = wave_sum(kq);
-      if (lane == 0) bg[tt * 4 + 2] = kq;
+      kq = row16_sum(kq);
+      if (sub == 0) bg[tt * 4 + 2] = kq;
     }
     __syncthreads();
     float o_m = 0.f;
-    for (int u = 0; u < nt; ++u) {
+#pragma unroll 4
+    for (int u = 0; u < nt; ++u) {   // unrolled: the LDS reads of the next tokens do not depend on the state
       const float beta = bg[u * 4], g = bg[u * 4 + 1], kq = bg[u * 4 + 2], v = vs[u * DR_COLS + col];
       float kk[NS];
-      float a = 0.f, b = 0.f;
+      float a2[2] = {0.f, 0.f}, b2[2] = {0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < NS; ++r) {
         kk[r] = ks[u * DP + r * 16 + sub];
-        a += S[r] * kk[r];
-        b += S[r] * qs[u * DP + r * 16 + sub];
+        a2[r & 1] += S[r] * kk[r];
+        b2[r & 1] += S[r] * qs[u * DP + r * 16 + sub];
       }
-      a = row16_sum(a);
-      b = row16_sum(b);
+      const float a = row16_sum(a2[0] + a2[1]);
+      const float b = row16_sum(b2[0] + b2[1]);
       const float uu = beta * (v - g * a);
 #pragma unroll
       for (int r = 0; r < NS; ++r) S[r] = g * S[r] + kk[r] * uu;
@@ -147,9 +175,12 @@ __global__ void __launch_bounds__(256) delta_finish_kernel(const float* __restri
   const int lane = threadIdx.x & 63;
   const long tok = r / H;
   const int h = (int)(r % H);
-  bool live = false;   // tokens of no sequence keep their zeros
+  bool live = false;   // tokens of no sequence (graph padding) become zeros
   for (int s = 0; s < S; ++s) live |= tok >= qstart[s] && tok < qstart[s] + qlen[s];
-  if (!live) return;
+  if (!live) {
+    for (int j = lane; j < dv; j += 64) stf(out + tok * ((long)H * dv) + (long)h * dv + j, 0.f);
+    return;
+  }
   const float* o = raw + r * dv;
   float ss = 0.f;
   for (int j = lane; j < dv; j += 64) ss += o[j] * o[j];

@@ -240,7 +240,7 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
                                                              const int* __restrict__ tile_seq,
                                                              const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
                                                              long ldg, u16* __restrict__ out, int H, int G, int d, int dv,
-                                                             int TQ) {
+                                                             int TQ, int splits, float* __restrict__ part) {
   constexpr int DS = SZ / 32, VB = SZ / 16, NKB = GM_KT / 16;
   constexpr int KSTR = SZ + 8, VSTR = GM_KT + 8, PSTR = GM_KT + 8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
@@ -310,8 +310,13 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
         pv_[f] = *reinterpret_cast<const uint4*>(vc + (((long)btr[(k0 >> 4) + pg] * G + g) * dv + j) * GM_BS + 8 * hf);
     }
   };
-  fetch(0);
-  for (int k0 = 0; k0 <= last; k0 += GM_KT) {
+  // small grids (decode steps) split a row's key tiles over `splits` workgroups; each leaves its
+  // running maximum, sum and unnormalised output in `part`, gqa_combine merges them
+  const int ntiles = last / GM_KT + 1;
+  const int kbeg = (int)((long)ntiles * blockIdx.z / splits) * GM_KT;
+  const int kend = (int)((long)ntiles * (blockIdx.z + 1) / splits) * GM_KT;   // exclusive
+  if (kbeg < kend) fetch(kbeg);
+  for (int k0 = kbeg; k0 < kend; k0 += GM_KT) {
     __syncthreads();   // the previous tile is consumed
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
@@ -321,7 +326,7 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
       const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8);
       *reinterpret_cast<uint4*>(vtr + j * VSTR + 8 * cc) = pv_[f];
     }
-    if (k0 + GM_KT <= last) fetch(k0 + GM_KT);   // the next tile's loads fly under this tile's products
+    if (k0 + GM_KT < kend) fetch(k0 + GM_KT);   // the next tile's loads fly under this tile's products
     __syncthreads();
     if (k0 > wave_last) continue;   // this wave's rows see nothing of the tile (the barriers above are uniform)
     f32x4 sacc[NKB];
@@ -388,6 +393,14 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
     const float lt = row16_add(l[i]);
     const int row = 16 * wave + 4 * g4 + i;
     if (row >= nrows) continue;
+    if (part) {
+      float* pr = part + ((((long)blockIdx.x * G + g) * splits + blockIdx.z) * GM_ROWS + row) * (dv + 2);
+      if (lr == 0) { pr[0] = m[i]; pr[1] = lt; }
+#pragma unroll
+      for (int cb = 0; cb < VB; ++cb)
+        if (16 * cb + lr < dv) pr[2 + 16 * cb + lr] = acc[cb][i];
+      continue;
+    }
     const long tok = q0 + tok0 + row / R;
     const int h = g * R + row % R;
     const float inv = 1.f / lt;
@@ -396,6 +409,38 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
       const int jx = 16 * cb + lr;
       if (jx >= dv) continue;
       float o = acc[cb][i] * inv;
+      if (gate) o *= 1.f / (1.f + expf(-bf2f(gate[tok * ldg + (long)h * dv + jx])));
+      out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
+    }
+  }
+}
+
+// merge the key splits of paged_gqa_mfma: one wave per (tile, kv head, row)
+__global__ void __launch_bounds__(256) gqa_combine_kernel(const float* __restrict__ part, int splits,
+                                                          const int* __restrict__ qstart, const int* __restrict__ qlen,
+                                                          const int* __restrict__ tile_seq,
+                                                          const int* __restrict__ tile_tok0, const u16* __restrict__ gate,
+                                                          long ldg, u16* __restrict__ out, int H, int G, int dv, int TQ) {
+  const int s = tile_seq[blockIdx.x];
+  const int n = qlen[s], tok0 = tile_tok0[blockIdx.x];
+  if (n <= 0 || tok0 >= n) return;
+  const int g = blockIdx.y, R = H / G;
+  const int nrows = min(TQ, n - tok0) * R;
+  const int lane = threadIdx.x & 63;
+  for (int row = blockIdx.z * 4 + (threadIdx.x >> 6); row < nrows; row += 4 * gridDim.z) {
+    const float* pr = part + (((long)blockIdx.x * G + g) * splits * GM_ROWS + row) * (dv + 2);
+    const long zs = (long)GM_ROWS * (dv + 2);
+    float M = -INFINITY;
+    for (int z = 0; z < splits; ++z) M = fmaxf(M, pr[z * zs]);
+    float L = 0.f;
+    for (int z = 0; z < splits; ++z) L += pr[z * zs + 1] * (pr[z * zs] > -INFINITY ? expf(pr[z * zs] - M) : 0.f);
+    const long tok = qstart[s] + tok0 + row / R;
+    const int h = g * R + row % R;
+    for (int jx = lane; jx < dv; jx += 64) {
+      float o = 0.f;
+      for (int z = 0; z < splits; ++z)
+        if (pr[z * zs] > -INFINITY) o += pr[z * zs + 2 + jx] * expf(pr[z * zs] - M);
+      o /= L;
       if (gate) o *= 1.f / (1.f + expf(-bf2f(gate[tok * ldg + (long)h * dv + jx])));
       out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);
     }
@@ -468,23 +513,31 @@ extern "C" int dllm_gqa_tile_tokens(int H, int G, int mfma) {
 extern "C" int dllm_paged_gqa(const void* q, const void* kc, const void* vc, int f32, const int* bt, int bt_ld, int BSZ,
                               const int* qstart, const int* qlen, const int* ctx, const int* tile_seq, const int* tile_tok0,
                               int n_tiles, const void* gate, long ldg, void* out, int H, int G, int d, int dv, int mfma,
-                              hipStream_t st) {
+                              int splits, float* part, hipStream_t st) {
   if (n_tiles <= 0) return 0;
   if (G < 1 || H % G || dv > 256 || d < 1) return -1;
   if (mfma) {
     if (!dllm_gqa_mfma_ok(f32, H, G, d, dv, BSZ)) return -1;
     const int sz = d > dv ? d : dv;
-    const dim3 grid(n_tiles, G);
+    if (splits < 1 || (splits > 1 && !part)) return -1;
+    const dim3 grid(n_tiles, G, splits);
     const int TQ = dllm_gqa_tile_tokens(H, G, 1);
+    float* pp = splits > 1 ? part : nullptr;
 #define GQM(SZ)                                                                                                          \
   do {                                                                                                                   \
     const long lds = gqa_mfma_lds(SZ);                                                                                   \
     ENSURE_LDS(paged_gqa_mfma_kernel<SZ>, lds);                                                                          \
     hipLaunchKernelGGL(paged_gqa_mfma_kernel<SZ>, grid, dim3(256), lds, st, (const u16*)q, (const u16*)kc, (const u16*)vc, bt, \
-                       bt_ld, qstart, qlen, ctx, tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, d, dv, TQ); \
+                       bt_ld, qstart, qlen, ctx, tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, d, dv, TQ, \
+                       splits, pp);                                                                                      \
   } while (0)
     if (sz <= 64) GQM(64); else if (sz <= 128) GQM(128); else GQM(256);
 #undef GQM
+    if (pp) {
+      const int rows = (TQ * (H / G) < GM_ROWS ? TQ * (H / G) : GM_ROWS);
+      hipLaunchKernelGGL(gqa_combine_kernel, dim3(n_tiles, G, (rows + 3) / 4), dim3(256), 0, st, pp, splits, qstart, qlen,
+                         tile_seq, tile_tok0, (const u16*)gate, ldg, (u16*)out, H, G, dv, TQ);
+    }
     return (int)hipGetLastError();
   }
   int KT = 64;

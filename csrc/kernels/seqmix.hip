@@ -587,7 +587,10 @@ __global__ void __launch_bounds__(256) heads_norm_gate_kernel(const float* __res
   const long tok = blockIdx.x;
   bool live = false;
   for (int s = 0; s < S; ++s) live |= tok >= qstart[s] && tok < qstart[s] + qlen[s];
-  if (!live) return;     // the whole workgroup: rows of no sequence keep their zeros
+  if (!live) {           // the whole workgroup: rows of no sequence (graph padding) become zeros
+    for (int j = threadIdx.x; j < n; j += 256) stf(out + tok * n + j, 0.f);
+    return;
+  }
   const float* o = raw + tok * n;
   float ss = 0.f;
   for (int j = threadIdx.x; j < n; j += 256) ss += o[j] * o[j];

@@ -112,7 +112,8 @@ def sedopel_kernel_rooflines(z: dict, T: int = 4096, B: int = 64, ctx: int = 204
         ts, tt = meta.latent_tiles(1, dev, seqmix.gqa_tokens_per_tile(H, G, mfma))
         gate = proj[:, (H + G) * d + G * dv:]
         rec(f"attention_{tag}",
-            _timed(lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, gate, mfma), 3),
+            _timed(lambda: seqmix.paged_gqa_attention(q, kc, vc, bt, qstart, qlen, cx, ts, tt, gate, mfma,
+                                                      seqmix.gqa_splits(int(ts.numel()), G, max(cxl)) if mfma else 1), 3),
             sum(cxl) * G * (d + dv) * 2 + n * H * (d + 2 * dv) * 2, keys * H * 2 * (d + dv), PEAK_BF16)
         # lightning attention
         Hl, dl, dvl = z["l_heads"], z["l_dim"], z["l_vdim"]

@@ -392,8 +392,9 @@ class HybridModel:
         mfma = seqmix.gqa_use_mfma(q, a.heads, a.kv_heads, a.dim, a.vdim, k_cache.shape[2])
         ts, tt = meta.latent_tiles(1, self.device, seqmix.gqa_tokens_per_tile(a.heads, a.kv_heads, mfma))
         gate = proj[:, nl - a.heads * a.vdim:nl]
+        splits = seqmix.gqa_splits(int(ts.numel()), a.kv_heads, meta.max_ctx) if mfma else 1
         lo = seqmix.paged_gqa_attention(q, k_cache, v_cache, meta.block_tables, meta.qstart, meta.qlen, meta.ctx, ts, tt,
-                                        gate, mfma)
+                                        gate, mfma, splits)
         ro = seqmix.lightning_attention(proj[:, nl:], b.heads, b.dim, b.vdim, L["decay"], state, eps, L["rnorm"],
                                         meta.qstart, meta.qlen, meta.ctx, meta.state_rows)
         return _mm(lo, L["lo"]), _mm(ro, L["ro"])

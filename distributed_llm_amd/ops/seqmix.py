@@ -253,23 +253,41 @@ def attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, 
     if ext is None:
         return ref.attn_prep(proj, heads, kv_heads, dim, vdim, cos_sin, rot_dims, eps, qscale, positions, slots,
                              k_cache, v_cache)
-    q = torch.zeros((proj.shape[0], heads, dim), dtype=proj.dtype, device=proj.device)
+    q = torch.empty((proj.shape[0], heads, dim), dtype=proj.dtype, device=proj.device)     # every row is written
     ext.attn_prep(proj, int(heads), int(kv_heads), int(dim), int(vdim), cos_sin, int(rot_dims), float(eps), qscale,
                   positions, slots, k_cache, v_cache, q)
     return q
 
 
+GQA_SPLIT_TARGET = 512     # workgroups a small matrix-core attention grid is split up to (over keys)
+GQA_SPLIT_MAX = 16
+
+
+def gqa_splits(n_tiles: int, kv_heads: int, max_ctx: int) -> int:
+    """Key splits of a matrix-core attention launch: grids with few workgroups (decode steps at small
+    batch, short portions) split every row's 64-key tiles over up to ``GQA_SPLIT_MAX`` workgroups."""
+    tiles = (int(max_ctx) + 63) // 64 if max_ctx > 0 else GQA_SPLIT_MAX     # decode graphs: any context
+    return max(1, min(GQA_SPLIT_MAX, tiles, GQA_SPLIT_TARGET // max(1, n_tiles * kv_heads)))
+
+
 def paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0,
-                        gate: Optional[torch.Tensor] = None, mfma: bool = False) -> torch.Tensor:
+                        gate: Optional[torch.Tensor] = None, mfma: bool = False, splits: int = 1) -> torch.Tensor:
     """Causal softmax attention over paged keys / values of any head widths (f32 scores, online
     softmax), output times sigmoid(gate).  ``tile_seq`` / ``tile_tok0``: one entry per
-    ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence."""
+    ``gqa_tokens_per_tile(heads, kv_heads, mfma)`` new tokens of a sequence.  ``splits`` > 1
+    (matrix-core kernel): a row's keys are split over that many workgroups and merged."""
     ext = _native(q)
     if ext is None:
         return ref.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, gate)
-    out = torch.zeros((q.shape[0], q.shape[1] * v_cache.shape[2]), dtype=q.dtype, device=q.device)
+    dv = v_cache.shape[2]
+    out = torch.zeros((q.shape[0], q.shape[1] * dv), dtype=q.dtype, device=q.device)
+    splits = int(splits) if mfma else 1
+    part = None
+    if splits > 1:
+        part = torch.empty(int(tile_seq.numel()) * k_cache.shape[1] * splits * GQA_ROWS_MFMA * (dv + 2),
+                           dtype=torch.float32, device=q.device)
     ext.paged_gqa_attention(q, k_cache, v_cache, block_tables, qstart, qlen, ctx, tile_seq, tile_tok0, gate, out,
-                            bool(mfma))
+                            bool(mfma), splits, part)
     return out
 
 
@@ -284,12 +302,12 @@ def lightning_attention(qkvg, heads, dim, vdim, decay, state, eps, norm_w, qstar
     if ext is None:
         return ref.lightning_attention(qkvg, heads, dim, vdim, decay, state, eps, norm_w, qstart, qlen, ctx, rows)
     T = qkvg.shape[0]
-    out = torch.zeros((T, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)
+    out = torch.empty((T, heads * vdim), dtype=qkvg.dtype, device=qkvg.device)     # the finish kernel writes every row
     if chunked is None:
         chunked = T >= RETENTION_CHUNK_MIN * qstart.numel()
     if not chunked and retention_step_lds(dim, vdim) > 150 * 1024:
         chunked = True
-    raw = torch.zeros((T, heads, vdim), dtype=torch.float32, device=qkvg.device)
+    raw = torch.empty((T, heads, vdim), dtype=torch.float32, device=qkvg.device)    # read for live tokens only
     ext.lightning_attention(qkvg, int(heads), int(dim), int(vdim), decay, state, float(eps), norm_w, qstart, qlen, ctx,
                             rows, out, raw, bool(chunked))
     return out
@@ -311,7 +329,7 @@ def delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps
     if ext is None:
         return ref.delta_rule(qkv, gba, heads, kv_heads, dim, vdim, neg_a, dt_bias, norm_w, eps, state, qstart, qlen,
                               ctx, rows)
-    out = torch.zeros((qkv.shape[0], heads * vdim), dtype=qkv.dtype, device=qkv.device)
+    out = torch.empty((qkv.shape[0], heads * vdim), dtype=qkv.dtype, device=qkv.device)     # the finish kernel writes every row
     ext.delta_rule(qkv, gba, int(heads), int(kv_heads), int(dim), int(vdim), neg_a, dt_bias, norm_w, float(eps), state,
                    qstart, qlen, ctx, rows, out)
     return out

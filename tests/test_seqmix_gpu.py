@@ -233,7 +233,7 @@ def _pages(case, G, d, dv, dt, BSz=16):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES + [([40, 3], [90, 130])])
-@pytest.mark.parametrize("H,G,d,dv,rot", [(4, 2, 16, 8, 8), (6, 3, 96, 48, 24), (3, 3, 40, 72, 40), (34, 2, 8, 5, 0),
+@pytest.mark.parametrize("H,G,d,dv,rot", [(4, 2, 16, 8, 8), (6, 2, 88, 56, 20), (3, 3, 40, 72, 40), (34, 2, 8, 5, 0),
                                           (8, 1, 64, 64, 32), (2, 1, 136, 200, 64)])
 def test_attn_prep_and_paged_gqa(dt, case, H, G, d, dv, rot):
     from distributed_llm_amd.models.llama import AttnMeta
@@ -255,8 +255,9 @@ def test_attn_prep_and_paged_gqa(dt, case, H, G, d, dv, rot):
     forms = [False] + ([True] if seqmix.gqa_use_mfma(q2, H, G, d, dv, 16) else [])
     for mfma in forms:
         ts, tt = meta.latent_tiles(1, DEV, seqmix.gqa_tokens_per_tile(H, G, mfma))
-        got = seqmix.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, ts, tt, gate, mfma).float()
-        torch.testing.assert_close(got, want, **tol(dt))
+        for splits in ((1, 2, 5) if mfma else (1,)):      # 5: more splits than some rows have key tiles
+            got = seqmix.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, ts, tt, gate, mfma, splits).float()
+            torch.testing.assert_close(got, want, **tol(dt))
 
 
 def test_paged_gqa_mfma_keeps_small_weights():
@@ -282,7 +283,7 @@ def test_paged_gqa_mfma_keeps_small_weights():
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES)
-@pytest.mark.parametrize("H,d,dv", [(2, 8, 6), (4, 64, 32), (1, 40, 130), (3, 128, 128)])
+@pytest.mark.parametrize("H,d,dv", [(2, 8, 6), (4, 48, 40), (1, 40, 130), (3, 128, 128)])
 @pytest.mark.parametrize("chunked", [False, True])
 def test_lightning_attention(dt, case, H, d, dv, chunked):
     torch.manual_seed(6)
@@ -300,7 +301,7 @@ def test_lightning_attention(dt, case, H, d, dv, chunked):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", CASES)
-@pytest.mark.parametrize("H,G,d,dv,K", [(4, 2, 8, 6, 3), (6, 3, 64, 32, 4), (1, 1, 20, 33, 1), (2, 1, 200, 18, 2), (2, 2, 128, 128, 4)])
+@pytest.mark.parametrize("H,G,d,dv,K", [(4, 2, 8, 6, 3), (6, 2, 72, 24, 5), (1, 1, 20, 33, 1), (2, 1, 200, 18, 2), (2, 2, 128, 128, 4)])
 def test_delta_rule_and_conv_refill(dt, case, H, G, d, dv, K):
     torch.manual_seed(7)
     T, qstart, qlen, ctx, rows, pos = batch(*case)
