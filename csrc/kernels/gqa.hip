@@ -226,6 +226,8 @@ __device__ __forceinline__ float row16_add(float v) {
 }
 
 constexpr int GM_ROWS = 64, GM_KT = 64, GM_BS = 16;   // rows per workgroup, keys per tile, keys per page
+typedef float f32x2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 
 // SZ >= max(d, dv) in {64, 128, 256}: d is walked in SZ / 32 MFMA steps, dv in SZ / 16 column blocks
 // (steps and blocks past the real widths are skipped).  d % 8 == 0 (16-byte key rows).
@@ -285,6 +287,8 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
 #pragma unroll
   for (int cb = 0; cb < VB; ++cb) acc[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int wave_last = 16 * wave < nrows ? p0 + tok0 + (min(16 * wave + 15, nrows - 1)) / R : -1;
+  // the oldest row of the wave; idle rows (past nrows) are masked, so a wave that has any never skips the mask
+  const int wave_first = 16 * wave + 15 < nrows ? p0 + tok0 + (16 * wave) / R : -1;
   const int last = p0 + tok0 + nq - 1;   // the newest key any row sees
   const int* btr = bt + (long)s * bt_ld;
   constexpr int KCH = SZ / 8;            // 16-byte chunks of a staged key row
@@ -292,22 +296,33 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
   // Score block kb, column lr stands for key 4 lr + kb of the tile (K rows are staged in that order),
   // so a lane's four blocks are four neighbouring keys and its weights leave as 8-byte vectors.
   uint4 pk_[NF], pv_[NF];
+  // A thread moves the same (key, chunk) and (dim, page, half) of every tile (tiles start at multiples
+  // of 64 keys), so only the page ids change from tile to tile: offsets inside a page are kept.
+  long koff[NF], voff[NF];
+  int kkey[NF], vpg[NF];
+  bool kon[NF], von[NF];
+  const long kpage = (long)G * GM_BS * d, vpage = (long)G * dv * GM_BS;
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    const int e = tid + 256 * f;
+    const int kk = e / KCH, c = (e % KCH) * 8;
+    kkey[f] = kk;
+    kon[f] = c < d;
+    koff[f] = ((long)g * GM_BS + (kk & 15)) * d + c;
+    const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8);
+    vpg[f] = cc >> 1;
+    von[f] = j < dv;
+    voff[f] = ((long)g * dv + j) * GM_BS + 8 * (cc & 1);
+  }
   auto fetch = [&](int k0) {
     const int nk = min(GM_KT, last + 1 - k0);
+    const int* pg = btr + (k0 >> 4);
 #pragma unroll
     for (int f = 0; f < NF; ++f) {
-      const int e = tid + 256 * f;
-      const int kk = e / KCH, c = (e % KCH) * 8;
       pk_[f] = make_uint4(0u, 0u, 0u, 0u);
-      if (kk < nk && c < d) {
-        const int pk = k0 + kk;
-        pk_[f] = *reinterpret_cast<const uint4*>(kc + (((long)btr[pk >> 4] * G + g) * GM_BS + (pk & 15)) * d + c);
-      }
-      // values: a page holds [dv][16 keys]; entry (dim j, page pg, half hf) is 8 keys = 16 bytes
-      const int j = e / (GM_KT / 8), cc = e % (GM_KT / 8), pg = cc >> 1, hf = cc & 1;
+      if (kon[f] && kkey[f] < nk) pk_[f] = *reinterpret_cast<const uint4*>(kc + pg[kkey[f] >> 4] * kpage + koff[f]);
       pv_[f] = make_uint4(0u, 0u, 0u, 0u);
-      if (j < dv && 16 * pg < nk)
-        pv_[f] = *reinterpret_cast<const uint4*>(vc + (((long)btr[(k0 >> 4) + pg] * G + g) * dv + j) * GM_BS + 8 * hf);
+      if (von[f] && 16 * vpg[f] < nk) pv_[f] = *reinterpret_cast<const uint4*>(vc + pg[vpg[f]] * vpage + voff[f]);
     }
   };
   // small grids (decode steps) split a row's key tiles over `splits` workgroups; each leaves its
@@ -344,38 +359,46 @@ __global__ void __launch_bounds__(256) paged_gqa_mfma_kernel(const u16* __restri
     }
     float alpha[4];
     const int key0 = k0 + 4 * lr;
+    // a tile below the wave's oldest row needs no mask (wave-uniform)
+    const bool full = k0 + GM_KT - 1 <= wave_first;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float mx = -INFINITY;
+      float sv[NKB];
 #pragma unroll
-      for (int kb = 0; kb < NKB; ++kb) mx = fmaxf(mx, key0 + kb <= rpos[i] ? sacc[kb][i] : -INFINITY);
+      for (int kb = 0; kb < NKB; ++kb) sv[kb] = (full || key0 + kb <= rpos[i]) ? sacc[kb][i] : -INFINITY;
+      float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       mx = row16_max(mx);
       const float mn = fmaxf(m[i], mx);
       const bool any = mn > -INFINITY;
       alpha[i] = any ? __expf(m[i] - mn) : 1.f;   // m = -inf before the first visible key: 0, and acc, l are 0
       m[i] = mn;
       l[i] *= alpha[i];
-      uint32_t hi[NKB], lo[NKB];
+      float p[NKB];
 #pragma unroll
       for (int kb = 0; kb < NKB; ++kb) {
-        const float p = (any && key0 + kb <= rpos[i]) ? __expf(sacc[kb][i] - mn) : 0.f;
-        l[i] += p;
-        // p is in [0, 1]: round to nearest even without the special cases
-        uint32_t u = __float_as_uint(p);
-        u = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-        hi[kb] = u;
-        uint32_t w = __float_as_uint(p - __uint_as_float(u << 16));
-        lo[kb] = (w + 0x7fffu + ((w >> 16) & 1u)) >> 16;
+        p[kb] = any ? __expf(sv[kb] - mn) : 0.f;   // exp(-inf) = 0 for masked keys
+        l[i] += p[kb];
       }
-      *reinterpret_cast<uint2*>(phi + (4 * g4 + i) * PSTR + 4 * lr) = make_uint2(hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16));
-      *reinterpret_cast<uint2*>(plo + (4 * g4 + i) * PSTR + 4 * lr) = make_uint2(lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16));
+      // p = hi + lo with both parts bf16 (the packed conversions round to nearest even)
+      const uint32_t h01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2v{p[0], p[1]}, bf16x2v));
+      const uint32_t h23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2v{p[2], p[3]}, bf16x2v));
+      const f32x2v r01 = {p[0] - __uint_as_float(h01 << 16), p[1] - __uint_as_float(h01 & 0xffff0000u)};
+      const f32x2v r23 = {p[2] - __uint_as_float(h23 << 16), p[3] - __uint_as_float(h23 & 0xffff0000u)};
+      const uint32_t l01 = __builtin_bit_cast(uint32_t, __builtin_convertvector(r01, bf16x2v));
+      const uint32_t l23 = __builtin_bit_cast(uint32_t, __builtin_convertvector(r23, bf16x2v));
+      *reinterpret_cast<uint2*>(phi + (4 * g4 + i) * PSTR + 4 * lr) = make_uint2(h01, h23);
+      *reinterpret_cast<uint2*>(plo + (4 * g4 + i) * PSTR + 4 * lr) = make_uint2(l01, l23);
     }
     __builtin_amdgcn_wave_barrier();   // the patch is this wave's own: its LDS writes are in order before the reads
+    // once the running maxima have settled no row of the wave rescales: skip the sweep over the sums
+    const bool rescale = __any(alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f);
 #pragma unroll
     for (int cb = 0; cb < VB; ++cb) {
       if (cb * 16 >= dv) continue;
+      if (rescale) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc[cb][i] *= alpha[i];
+        for (int i = 0; i < 4; ++i) acc[cb][i] *= alpha[i];
+      }
       const u16* bp = vtr + (16 * cb + lr) * VSTR + 8 * g4;
 #pragma unroll
       for (int ks = 0; ks < GM_KT; ks += 32) {
