@@ -453,16 +453,24 @@ __global__ void __launch_bounds__(256) gqa_combine_kernel(const float* __restric
   for (int row = blockIdx.z * 4 + (threadIdx.x >> 6); row < nrows; row += 4 * gridDim.z) {
     const float* pr = part + (((long)blockIdx.x * G + g) * splits * GM_ROWS + row) * (dv + 2);
     const long zs = (long)GM_ROWS * (dv + 2);
-    float M = -INFINITY;
-    for (int z = 0; z < splits; ++z) M = fmaxf(M, pr[z * zs]);
-    float L = 0.f;
-    for (int z = 0; z < splits; ++z) L += pr[z * zs + 1] * (pr[z * zs] > -INFINITY ? expf(pr[z * zs] - M) : 0.f);
+    // lane z holds split z's maximum and sum (splits <= 64); weights travel by shuffles
+    const float mz = lane < splits ? pr[lane * zs] : -INFINITY;
+    const float lz = lane < splits ? pr[lane * zs + 1] : 0.f;
+    const float M = wave_max(mz);
+    const float wz = mz > -INFINITY ? expf(mz - M) : 0.f;
+    const float L = wave_sum(lz * wz);
     const long tok = qstart[s] + tok0 + row / R;
     const int h = g * R + row % R;
-    for (int jx = lane; jx < dv; jx += 64) {
+    for (int j0 = 0; j0 < dv; j0 += 64) {     // every lane stays in the loop: the shuffles read all lanes
+      const int jx = j0 + lane;
+      const bool on = jx < dv;
       float o = 0.f;
-      for (int z = 0; z < splits; ++z)
-        if (pr[z * zs] > -INFINITY) o += pr[z * zs + 2 + jx] * expf(pr[z * zs] - M);
+#pragma unroll 4
+      for (int z = 0; z < splits; ++z) {
+        const float w = __shfl(wz, z, 64);
+        if (on) o += pr[z * zs + 2 + jx] * w;
+      }
+      if (!on) continue;
       o /= L;
       if (gate) o *= 1.f / (1.f + expf(-bf2f(gate[tok * ldg + (long)h * dv + jx])));
       out[tok * ((long)H * dv) + (long)h * dv + jx] = f2bf(o);

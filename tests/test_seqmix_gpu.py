@@ -255,7 +255,7 @@ def test_attn_prep_and_paged_gqa(dt, case, H, G, d, dv, rot):
     forms = [False] + ([True] if seqmix.gqa_use_mfma(q2, H, G, d, dv, 16) else [])
     for mfma in forms:
         ts, tt = meta.latent_tiles(1, DEV, seqmix.gqa_tokens_per_tile(H, G, mfma))
-        for splits in ((1, 2, 5) if mfma else (1,)):      # 5: more splits than some rows have key tiles
+        for splits in ((1, 2, 7) if mfma else (1,)):      # 7: more splits than some rows have key tiles, and than value dims
             got = seqmix.paged_gqa_attention(q2, kc2, vc2, bt, qstart, qlen, ctx, ts, tt, gate, mfma, splits).float()
             torch.testing.assert_close(got, want, **tol(dt))
 
