@@ -15,7 +15,7 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 KERNELS = ["attention.hip", "gemv.hip", "skinny_gemm.hip", "sampling.hip", "moe.hip",
-           "flash_prefill.hip", "tgemm.hip", "encoder.hip"]
+           "flash_prefill.hip", "tgemm.hip", "encoder.hip", "gqa.hip", "delta.hip"]
 # measured exceptions (bytes/lane allowed): the d=64 flash prefill at 4 waves per SIMD (128-VGPR cap,
 # two workgroups per CU) keeps ~5 values in scratch around the chunk loop and is still 1.14-1.17x
 # faster than the spill-free one-workgroup build (profiles/r2_flash_prefill_microbench.md)
