@@ -38,7 +38,9 @@ constexpr int DR_COLS = 16; // value columns per workgroup
 
 // NS: state entries per lane; lane `sub` of a column owns dims sub * NS .. sub * NS + NS - 1, kept in
 // LDS at [r * 16 + sub] so that the 16 lanes of a row read consecutive words.
-template <typename T, int NS>
+// VL (bf16, rows of whole 16-byte vectors): q / k rows are fetched as 16-byte vectors, 8 dims a thread,
+// instead of NS scattered 2-byte loads a thread.
+template <typename T, int NS, bool VL>
 __global__ void __launch_bounds__(256) delta_rule_kernel(const T* __restrict__ qkv, long ldq, const T* __restrict__ gba,
                                                          long ldg, int H, int G, int d, int dv,
                                                          const float* __restrict__ neg_a,
@@ -68,18 +70,36 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(const T* __restrict__ q
   const float na = neg_a[h], dtb = dt_bias[h], qscale = 1.f / sqrtf((float)d);
   // a group's inputs are fetched into registers one group ahead, so their latency hides under the
   // previous group's recurrence: NS entries of q and of k, one of v, and (lanes < 16) the two logits
-  float pq[NS], pk[NS], pv = 0.f, pb = 0.f, pa = 0.f;
+  constexpr int NFV = (NS + 7) / 8;          // 16-byte chunks of q (and of k) a thread moves per group: 16 rows of d / 8
+  float pq[VL ? 1 : NS], pk[VL ? 1 : NS], pv = 0.f, pb = 0.f, pa = 0.f;
+  uint4 vq[VL ? NFV : 1], vk[VL ? NFV : 1];
+  const int dch = d >> 3;                    // chunks per row (VL: d % 8 == 0)
   auto fetch = [&](int t0) {
     const int nt = min(DR_TT, n - t0);
+    if constexpr (VL) {
 #pragma unroll
-    for (int r = 0; r < NS; ++r) {
-      const int e = tid + 256 * r;
-      const int tt = e / DP, c = e % DP;       // c = r' * 16 + sub'  ->  dim sub' * NS + r'
-      const int i = (c & 15) * NS + (c >> 4);
-      const bool okx = tt < nt && i < d;
-      const T* row = qkv + (long)(q0 + t0 + (okx ? tt : 0)) * ldq;
-      pq[r] = okx ? ldf(row + oq + i) : 0.f;
-      pk[r] = okx ? ldf(row + ok + i) : 0.f;
+      for (int f = 0; f < NFV; ++f) {
+        const int e = tid + 256 * f;
+        const int tt = e / dch, ch = e - tt * dch;
+        vq[f] = make_uint4(0u, 0u, 0u, 0u);
+        vk[f] = make_uint4(0u, 0u, 0u, 0u);
+        if (tt < nt) {
+          const u16* row = reinterpret_cast<const u16*>(qkv) + (long)(q0 + t0 + tt) * ldq + 8 * ch;
+          vq[f] = *reinterpret_cast<const uint4*>(row + oq);
+          vk[f] = *reinterpret_cast<const uint4*>(row + ok);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < NS; ++r) {
+        const int e = tid + 256 * r;
+        const int tt = e / DP, c = e % DP;       // c = r' * 16 + sub'  ->  dim sub' * NS + r'
+        const int i = (c & 15) * NS + (c >> 4);
+        const bool okx = tt < nt && i < d;
+        const T* row = qkv + (long)(q0 + t0 + (okx ? tt : 0)) * ldq;
+        pq[r] = okx ? ldf(row + oq + i) : 0.f;
+        pk[r] = okx ? ldf(row + ok + i) : 0.f;
+      }
     }
     {
       const int tt = tid / DR_COLS, c = tid % DR_COLS;
@@ -91,14 +111,37 @@ __global__ void __launch_bounds__(256) delta_rule_kernel(const T* __restrict__ q
       pa = ldf(row + oa);
     }
   };
+  if constexpr (VL) {   // dims past d (the lanes' padding) are never written again: zero them once
+    for (int e = tid; e < DR_TT * DP; e += 256) { qs[e] = 0.f; ks[e] = 0.f; }
+  }
   fetch(0);
   for (int t0 = 0; t0 < n; t0 += DR_TT) {
     const int nt = min(DR_TT, n - t0);
     __syncthreads();   // the previous group is consumed
+    if constexpr (VL) {
 #pragma unroll
-    for (int r = 0; r < NS; ++r) {
-      qs[tid + 256 * r] = pq[r];
-      ks[tid + 256 * r] = pk[r];
+      for (int f = 0; f < NFV; ++f) {
+        const int e = tid + 256 * f;
+        const int tt = e / dch, ch = e - tt * dch;
+        if (tt < DR_TT) {
+          float q8[8], k8[8];
+          unpack8(vq[f], q8);
+          unpack8(vk[f], k8);
+#pragma unroll
+          for (int x = 0; x < 8; ++x) {
+            const int i = 8 * ch + x;          // dim i = sub * NS + r lies at [r * 16 + sub]
+            const int pos = tt * DP + (i % NS) * 16 + i / NS;
+            qs[pos] = q8[x];
+            ks[pos] = k8[x];
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < NS; ++r) {
+        qs[tid + 256 * r] = pq[r];
+        ks[tid + 256 * r] = pk[r];
+      }
     }
     vs[tid] = pv;
     if (tid < nt) {
@@ -192,11 +235,11 @@ __global__ void __launch_bounds__(256) delta_finish_kernel(const float* __restri
   }
 }
 
-template <typename T>
+template <typename T, bool VL>
 int launch_delta(int ns, dim3 g, hipStream_t st, const T* qkv, long ldq, const T* gba, long ldg, int H, int G, int d, int dv,
                  const float* neg_a, const float* dt_bias, float* state, const int* qstart, const int* qlen, const int* ctx,
                  const int* rows, float* raw) {
-#define DELTA(NS) hipLaunchKernelGGL((delta_rule_kernel<T, NS>), g, dim3(256), 0, st, qkv, ldq, gba, ldg, H, G, d, dv, neg_a, dt_bias, state, qstart, qlen, ctx, rows, raw)
+#define DELTA(NS) hipLaunchKernelGGL((delta_rule_kernel<T, NS, VL>), g, dim3(256), 0, st, qkv, ldq, gba, ldg, H, G, d, dv, neg_a, dt_bias, state, qstart, qlen, ctx, rows, raw)
   if (ns <= 1) DELTA(1); else if (ns <= 2) DELTA(2); else if (ns <= 4) DELTA(4); else if (ns <= 8) DELTA(8); else DELTA(16);
 #undef DELTA
   return (int)hipGetLastError();
@@ -218,13 +261,19 @@ extern "C" int dllm_delta_rule(const void* qkv, long ldq, const void* gba, long 
   const dim3 gf((unsigned)((rows_total + 3) / 4));
   int rc;
   if (f32) {
-    rc = launch_delta<float>(ns, g, st, (const float*)qkv, ldq, (const float*)gba, ldg, H, G, d, dv, neg_a, dt_bias, state,
-                             qstart, qlen, ctx, rows, raw);
+    rc = launch_delta<float, false>(ns, g, st, (const float*)qkv, ldq, (const float*)gba, ldg, H, G, d, dv, neg_a, dt_bias,
+                                    state, qstart, qlen, ctx, rows, raw);
     hipLaunchKernelGGL(delta_finish_kernel<float>, gf, dim3(256), 0, st, raw, (const float*)gba, ldg, H, dv, norm_w, eps,
                        qstart, qlen, S, (float*)out, rows_total);
   } else {
-    rc = launch_delta<u16>(ns, g, st, (const u16*)qkv, ldq, (const u16*)gba, ldg, H, G, d, dv, neg_a, dt_bias, state, qstart,
-                           qlen, ctx, rows, raw);
+    // 16-byte row vectors: every q / k head starts on a 16-byte boundary of a 16-byte aligned row
+    const bool vl = d % 8 == 0 && ldq % 8 == 0 && ((uintptr_t)qkv & 15) == 0;
+    if (vl)
+      rc = launch_delta<u16, true>(ns, g, st, (const u16*)qkv, ldq, (const u16*)gba, ldg, H, G, d, dv, neg_a, dt_bias, state,
+                                   qstart, qlen, ctx, rows, raw);
+    else
+      rc = launch_delta<u16, false>(ns, g, st, (const u16*)qkv, ldq, (const u16*)gba, ldg, H, G, d, dv, neg_a, dt_bias, state,
+                                    qstart, qlen, ctx, rows, raw);
     hipLaunchKernelGGL(delta_finish_kernel<u16>, gf, dim3(256), 0, st, raw, (const u16*)gba, ldg, H, dv, norm_w, eps, qstart,
                        qlen, S, (u16*)out, rows_total);
   }
