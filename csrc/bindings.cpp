@@ -50,8 +50,8 @@ int dllm_moe_ffn(const void*, long, long, int, const int*, const float*, int, in
                  int*, void*, float*, void*, int, hipStream_t);
 int dllm_rms_rows(const void*, long, int, const float*, void*, long, int, int, int, float, hipStream_t);
 int dllm_norm_resadd(const void*, long, int, const float*, float*, void*, int, int, float, hipStream_t);
-int dllm_conv_silu(const void*, long, int, const float*, const float*, const void*, const int*, const int*, const int*,
-                   const int*, void*, int, int, int, int, hipStream_t);
+int dllm_conv_silu(const void*, long, int, const float*, const float*, void*, const int*, const int*, const int*,
+                   const int*, void*, int, int, int, int, int, hipStream_t);
 int dllm_selective_scan(const void*, const void*, int, const float*, const float*, const void*, long, int, const float*,
                         const void*, long, float*, void*, int, const int*, const int*, const int*, const int*, void*, int,
                         int, int, hipStream_t);
@@ -1359,7 +1359,7 @@ void norm_resadd(torch::Tensor y, torch::Tensor w, double eps, torch::Tensor x, 
 }
 
 void causal_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor b, torch::Tensor state, torch::Tensor qstart,
-                      torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor y) {
+                      torch::Tensor qlen, torch::Tensor ctx, torch::Tensor rows, torch::Tensor y, bool refill) {
   const bool f = act_f32(x, "x");
   check_rows2d(x, "x");
   check_f32(w, "w");
@@ -1375,7 +1375,7 @@ void causal_conv_silu(torch::Tensor x, torch::Tensor w, torch::Tensor b, torch::
               "y [T, C]");
   auto m = seq_meta(qstart, qlen, ctx, rows, state.size(0));
   ok(dllm_conv_silu(x.data_ptr(), x.stride(0), f, w.data_ptr<float>(), b.data_ptr<float>(), state.data_ptr(), m.qstart,
-                    m.qlen, m.ctx, m.rows, y.data_ptr(), T, m.S, C, K, stream()),
+                    m.qlen, m.ctx, m.rows, y.data_ptr(), T, m.S, C, K, (int)refill, stream()),
      "causal_conv_silu");
 }
 
@@ -1779,7 +1779,8 @@ void latent_attention(torch::Tensor qa, torch::Tensor q, int64_t dim, int64_t ro
 PYBIND11_MODULE(_hip_kernels, m) {
   m.def("rms_rows", &rms_rows);
   m.def("norm_resadd", &norm_resadd);
-  m.def("causal_conv_silu", &causal_conv_silu);
+  m.def("causal_conv_silu", &causal_conv_silu, py::arg("x"), py::arg("w"), py::arg("b"), py::arg("state"), py::arg("qstart"),
+        py::arg("qlen"), py::arg("ctx"), py::arg("rows"), py::arg("y"), py::arg("refill") = false);
   m.def("selective_scan", &selective_scan);
   m.def("retention", &retention, py::arg("qkvg"), py::arg("heads"), py::arg("dim"), py::arg("vdim"), py::arg("cos_sin"),
         py::arg("rot"), py::arg("decay"), py::arg("state"), py::arg("eps"), py::arg("positions"), py::arg("qstart"),

@@ -171,10 +171,10 @@ __global__ void __launch_bounds__(256) conv_refill_kernel(const T* __restrict__ 
 // ---------------------------------------------------------------- causal conv + SiLU
 template <typename T>
 __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ w,
-                                                        const float* __restrict__ b, const T* __restrict__ state,
+                                                        const float* __restrict__ b, const T* state,
                                                         const int* __restrict__ qstart, const int* __restrict__ qlen,
                                                         const int* __restrict__ ctx, const int* __restrict__ rows,
-                                                        T* __restrict__ y, int C, int K) {
+                                                        T* __restrict__ y, int C, int K, T* refill) {
   const int s = blockIdx.y;
   const int n = qlen[s];
   if (n <= 0) return;
@@ -194,6 +194,13 @@ __global__ void __launch_bounds__(256) conv_silu_kernel(const T* __restrict__ x,
       acc += w[c * K + k] * u;
     }
     stf(y + (long)(q0 + j) * C + c, silu_f(acc));
+  }
+  // decode steps (`refill` set; every sequence brings one token, which this thread alone has read
+  // the slot for): shift the slot's inputs by one and append the token's, in the same launch
+  if (refill && n == 1 && K > 1 && blockIdx.z == 0 && (threadIdx.x >> 6) == 0) {
+    T* sw = refill + (long)rows[s] * (K - 1) * C + c;
+    for (int k = 0; k + 1 < K - 1; ++k) stf(sw + (long)k * C, p0 > 0 ? ldf(sw + (long)(k + 1) * C) : 0.f);
+    stf(sw + (long)(K - 2) * C, ldf(x + (long)q0 * ldx + c));
   }
 }
 
@@ -716,17 +723,18 @@ extern "C" int dllm_conv_refill(const void* x, long ldx, int f32, void* conv, in
   return (int)hipGetLastError();
 }
 
-extern "C" int dllm_conv_silu(const void* x, long ldx, int f32, const float* w, const float* b, const void* state,
+// refill != 0: a step of single tokens; the kernel also moves each token's input into its slot
+extern "C" int dllm_conv_silu(const void* x, long ldx, int f32, const float* w, const float* b, void* state,
                               const int* qstart, const int* qlen, const int* ctx, const int* rows, void* y, int T,
-                              int S, int C, int K, hipStream_t st) {
+                              int S, int C, int K, int refill, hipStream_t st) {
   if (T <= 0 || S <= 0) return 0;
   if (K < 1 || K > 9) return -1;
   int gz = (T + 31) / 32;
   if (gz > 128) gz = 128;
   const dim3 g((C + 63) / 64, S, gz), blk(256);
   BY_T(f32,
-       hipLaunchKernelGGL(conv_silu_kernel<u16>, g, blk, 0, st, (const u16*)x, ldx, w, b, (const u16*)state, qstart, qlen, ctx, rows, (u16*)y, C, K),
-       hipLaunchKernelGGL(conv_silu_kernel<float>, g, blk, 0, st, (const float*)x, ldx, w, b, (const float*)state, qstart, qlen, ctx, rows, (float*)y, C, K))
+       hipLaunchKernelGGL(conv_silu_kernel<u16>, g, blk, 0, st, (const u16*)x, ldx, w, b, (const u16*)state, qstart, qlen, ctx, rows, (u16*)y, C, K, refill ? (u16*)state : nullptr),
+       hipLaunchKernelGGL(conv_silu_kernel<float>, g, blk, 0, st, (const float*)x, ldx, w, b, (const float*)state, qstart, qlen, ctx, rows, (float*)y, C, K, refill ? (float*)state : nullptr))
   return (int)hipGetLastError();
 }
 

@@ -373,8 +373,11 @@ class HybridModel:
         rows = meta.state_rows
         c = 2 * m.kv_heads * m.dim + m.heads * m.vdim
         proj = _mm(x, L["proj"])                                        # q | k | v | gate | beta | decay logits
-        qkv = seqmix.causal_conv_silu(proj, L["conv"], L["conv_b"], conv_state, meta.qstart, meta.qlen, meta.ctx, rows)
-        seqmix.conv_state_refill(proj, conv_state, meta.qstart, meta.qlen, meta.ctx, rows)
+        single = meta.host_qlen is None      # a decode step: the convolution refills its slots itself
+        qkv = seqmix.causal_conv_silu(proj, L["conv"], L["conv_b"], conv_state, meta.qstart, meta.qlen, meta.ctx, rows,
+                                      refill=single)
+        if not single:
+            seqmix.conv_state_refill(proj, conv_state, meta.qstart, meta.qlen, meta.ctx, rows)
         o = seqmix.delta_rule(qkv, proj[:, c:], m.heads, m.kv_heads, m.dim, m.vdim, L["neg_a"], L["dt_b"], L["hnorm"],
                               self.cfg.rms_eps, state, meta.qstart, meta.qlen, meta.ctx, rows)
         return _mm(o, L["o"])

@@ -44,13 +44,19 @@ def norm_resadd(y: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor,
     return x
 
 
-def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows) -> torch.Tensor:
+def causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, refill: bool = False) -> torch.Tensor:
+    """``refill``: the step brings at most one token per sequence (a decode step) and the kernel also
+    moves each token's input into its slot; otherwise the slot is left to ``conv_state_refill`` or
+    to the scan."""
     ext = _native(x)
     if ext is None:
-        return ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows)
+        y = ref.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows)
+        if refill:
+            ref.conv_state_refill(x, conv_state, qstart, qlen, ctx, rows)
+        return y
     # rows of no sequence (graph padding) stay zero, never stale memory
     y = torch.zeros((x.shape[0], w.shape[0]), dtype=x.dtype, device=x.device)
-    ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y)
+    ext.causal_conv_silu(x, w, b, conv_state, qstart, qlen, ctx, rows, y, bool(refill))
     return y
 
 

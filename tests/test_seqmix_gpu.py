@@ -321,3 +321,11 @@ def test_delta_rule_and_conv_refill(dt, case, H, G, d, dv, K):
     seqmix.conv_state_refill(proj, c1, qstart, qlen, ctx, rows)
     ref.conv_state_refill(proj, c2, qstart, qlen, ctx, rows)
     torch.testing.assert_close(c1.float(), c2.float(), atol=0, rtol=0)
+    if max(case[0]) <= 1:      # a step of single tokens: the convolution refills the slots in its own launch
+        w, b = torch.randn(C, K, device=DEV), torch.randn(C, device=DEV)
+        c3 = c1.clone()
+        y1 = seqmix.causal_conv_silu(proj, w, b, c3, qstart, qlen, ctx, rows, refill=True)
+        y2 = ref.causal_conv_silu(proj, w, b, c1, qstart, qlen, ctx, rows)
+        ref.conv_state_refill(proj, c1, qstart, qlen, ctx, rows)
+        torch.testing.assert_close(y1.float(), y2.float(), **tol(dt))
+        torch.testing.assert_close(c3.float(), c1.float(), atol=0, rtol=0)
