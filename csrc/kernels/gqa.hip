@@ -18,7 +18,7 @@
 //               mantissa through two MFMAs.  Key blocks above a wave's newest row are skipped.
 //
 // Cache layout: K [blocks, G, block, d], V [blocks, G, dv, block] (bf16 or f32 like the activations;
-// V is kept transposed inside its page because the weighted sum contracts over keys); every score,
+// V is kept transposed inside its page because the weighted sum runs over keys); every score,
 // weight and sum is f32.
 #include "common.h"
 

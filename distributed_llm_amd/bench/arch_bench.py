@@ -2,7 +2,7 @@
 and decode throughput through the engine, and the time of each mixer kernel against its roofline.
 
 ``python bench.py --arch-bench [--arch-design filevik|sedopel] [--arch-size s|m]`` (random weights,
-synthetic tokens).  The default bench workload and its JSON contract are untouched; this prints one
+synthetic tokens).  The default bench workload and its JSON line are untouched; this prints one
 JSON object of its own.
 
 The Sedopel stack alternates parallel layers (grouped-query softmax attention beside lightning
