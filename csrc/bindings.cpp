@@ -65,7 +65,7 @@ int dllm_retention_chunked(const void*, long, int, int, int, int, const float*, 
 int dllm_heads_norm_gate(const float*, const void*, long, int, long, int, const float*, float, const int*, const int*, int,
                          void*, long, hipStream_t);
 int dllm_resadd_norm(const void*, long, const void*, long, int, const float*, const float*, const float*, float*,
-                     const float*, void*, int, int, float, hipStream_t);
+                     const float*, void*, int, int, float, const float*, int, hipStream_t);
 int dllm_depth_mix(float*, const float*, int, long, int, const float*, void*, int, float, hipStream_t);
 int dllm_gelu_erf(const void*, void*, int, long, hipStream_t);
 int dllm_conv_refill(const void*, long, int, void*, int, int, const int*, const int*, const int*, const int*, int,
@@ -1489,11 +1489,23 @@ void lightning_attention(torch::Tensor qkvg, int64_t H, int64_t d, int64_t dv, t
 
 void resadd_norm(torch::Tensor a, c10::optional<torch::Tensor> b, c10::optional<torch::Tensor> wa,
                  c10::optional<torch::Tensor> wb, torch::Tensor w_post, double eps, torch::Tensor x,
-                 c10::optional<torch::Tensor> w_next, c10::optional<torch::Tensor> xn) {
+                 c10::optional<torch::Tensor> w_next, c10::optional<torch::Tensor> xn,
+                 c10::optional<torch::Tensor> stack, c10::optional<torch::Tensor> dw, int64_t dn) {
   const bool f = act_f32(a, "a");
   check_rows2d(a, "a");
   check_f32(w_post, "w_post");
   check_f32(x, "x");
+  const float* dwp = nullptr;
+  if (stack) {   // x must be slot dn - 1 of the stack; slot dn receives the weighted sum over depth
+    TORCH_CHECK(dw.has_value(), "depth weights");
+    check_f32(*stack, "stack");
+    check_f32(*dw, "depth weights");
+    TORCH_CHECK(stack->dim() == 3 && stack->is_contiguous() && dn >= 1 && dn < stack->size(0) && dw->numel() >= dn &&
+                    stack->size(1) == x.size(0) && stack->size(2) == x.size(1) &&
+                    x.data_ptr<float>() == stack->data_ptr<float>() + (dn - 1) * stack->size(1) * stack->size(2),
+                "stack [slots, T, H] with x its slot dn - 1, dn < slots");
+    dwp = dw->data_ptr<float>();
+  }
   TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && x.sizes() == a.sizes() && w_post.numel() == x.size(1),
               "x / a / w_post shapes");
   const void* bp = nullptr;
@@ -1524,7 +1536,7 @@ void resadd_norm(torch::Tensor a, c10::optional<torch::Tensor> b, c10::optional<
     }
   }
   ok(dllm_resadd_norm(a.data_ptr(), a.stride(0), bp, ldb, f, wap, wbp, w_post.data_ptr<float>(), x.data_ptr<float>(), wnp,
-                      xp, (int)x.size(0), (int)x.size(1), (float)eps, stream()),
+                      xp, (int)x.size(0), (int)x.size(1), (float)eps, dwp, (int)dn, stream()),
      "resadd_norm");
 }
 
@@ -1788,7 +1800,9 @@ PYBIND11_MODULE(_hip_kernels, m) {
   m.def("relu2_scale", &relu2_scale);
   m.def("dense_gate", &dense_gate);
   m.def("lightning_attention", &lightning_attention);
-  m.def("resadd_norm", &resadd_norm);
+  m.def("resadd_norm", &resadd_norm, py::arg("a"), py::arg("b"), py::arg("wa"), py::arg("wb"), py::arg("w_post"),
+        py::arg("eps"), py::arg("x"), py::arg("w_next"), py::arg("x_next"), py::arg("stack") = py::none(),
+        py::arg("depth_w") = py::none(), py::arg("depth_n") = 0);
   m.def("depth_mix", &depth_mix);
   m.def("gelu_erf", &gelu_erf);
   m.def("conv_state_refill", &conv_state_refill);

@@ -79,7 +79,8 @@ __global__ void __launch_bounds__(256) resadd_norm_kernel(const T* __restrict__ 
                                                           long ldb, const float* __restrict__ wa,
                                                           const float* __restrict__ wb, const float* __restrict__ w_post,
                                                           float* __restrict__ x, const float* __restrict__ w_next,
-                                                          T* __restrict__ xn, int H, float eps) {
+                                                          T* __restrict__ xn, int H, float eps,
+                                                          const float* __restrict__ dw, int dn, long TH) {
   __shared__ float red[16];
   extern __shared__ float yb[];   // [H]; entry i is touched by thread i % 256 only
   const long row = blockIdx.x;
@@ -107,8 +108,18 @@ __global__ void __launch_bounds__(256) resadd_norm_kernel(const T* __restrict__ 
   float* xr = x + row * (long)H;
   float sx = 0.f;
   for (int i = threadIdx.x; i < H; i += 256) {
-    const float v = xr[i] + yb[i] * ry * w_post[i];
+    float v = xr[i] + yb[i] * ry * w_post[i];
     xr[i] = v;
+    if (dw) {
+      // the layer ends here: x is slot dn - 1 of the f32 stack (slot 0 lies dn - 1 slots before it);
+      // the weighted sum over slots 0 .. dn - 1 goes to slot dn and on to the next norm
+      const float* p0 = xr + i - (long)(dn - 1) * TH;
+      float acc = 0.f;
+      for (int j = 0; j + 1 < dn; ++j) acc += dw[j] * p0[j * TH];
+      acc += dw[dn - 1] * v;
+      xr[i + TH] = acc;
+      v = acc;
+    }
     yb[i] = v;
     sx += v * v;
   }
@@ -669,20 +680,22 @@ extern "C" int dllm_norm_resadd(const void* y, long ldy, int f32, const float* w
   return (int)hipGetLastError();
 }
 
+// dw != null: x is slot dn - 1 of an f32 stack [slots][rows][H]; the launch also writes slot dn, the
+// sum over j < dn of dw[j] * slot j, and norms that for xn
 extern "C" int dllm_resadd_norm(const void* a, long lda, const void* b, long ldb, int f32, const float* wa, const float* wb,
                                 const float* w_post, float* x, const float* w_next, void* xn, int rows, int H, float eps,
-                                hipStream_t st) {
+                                const float* dw, int dn, hipStream_t st) {
   if (rows <= 0) return rows == 0 ? 0 : -1;
   const long lds = 4L * H;
   if (lds > 150 * 1024) return -2;
   if (f32) {
     ENSURE_LDS(resadd_norm_kernel<float>, lds);
     hipLaunchKernelGGL(resadd_norm_kernel<float>, dim3(rows), dim3(256), lds, st, (const float*)a, lda, (const float*)b, ldb, wa,
-                       wb, w_post, x, w_next, (float*)xn, H, eps);
+                       wb, w_post, x, w_next, (float*)xn, H, eps, dw, dn, (long)rows * H);
   } else {
     ENSURE_LDS(resadd_norm_kernel<u16>, lds);
     hipLaunchKernelGGL(resadd_norm_kernel<u16>, dim3(rows), dim3(256), lds, st, (const u16*)a, lda, (const u16*)b, ldb, wa, wb,
-                       w_post, x, w_next, (u16*)xn, H, eps);
+                       w_post, x, w_next, (u16*)xn, H, eps, dw, dn, (long)rows * H);
   }
   return (int)hipGetLastError();
 }

@@ -481,10 +481,9 @@ class HybridModel:
                     a, pair, post = y, {}, L["norm2b"]
                 else:
                     post = L["norm1b"]
-                if X is not None:
-                    seqmix.resadd_norm(a, post, eps, x, **pair)
+                if X is not None:     # ... and the layer's weighted sum over depth
                     h = torch.empty((T, W), dtype=self.dtype, device=x.device)
-                    x = seqmix.depth_mix(X, L["dwa"], i + 2, nxt, eps, h)
+                    x = seqmix.resadd_norm(a, post, eps, x, nxt, h, depth=(X, L["dwa"], i + 2), **pair)
                 else:
                     h = torch.empty((T, W), dtype=self.dtype, device=x.device)
                     seqmix.resadd_norm(a, post, eps, x, nxt, h, **pair)

@@ -197,15 +197,24 @@ def dense_gate(ids, wts, E) -> torch.Tensor:
 def resadd_norm(a: torch.Tensor, w_post: torch.Tensor, eps: float, x: torch.Tensor,
                 w_next: Optional[torch.Tensor] = None, x_next: Optional[torch.Tensor] = None,
                 b: Optional[torch.Tensor] = None, wa: Optional[torch.Tensor] = None,
-                wb: Optional[torch.Tensor] = None) -> torch.Tensor:
+                wb: Optional[torch.Tensor] = None, depth: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None
+                ) -> torch.Tensor:
     """The tail of a sublayer in one launch: ``x += rmsnorm(y) * w_post`` on the f32 stream, where y
     is the sublayer's output ``a`` or, for two mixers side by side, ``(rmsnorm(a) wa + rmsnorm(b) wb) / 2``;
-    ``x_next`` (the model dtype) receives ``rmsnorm(x) * w_next``, the next sublayer's input."""
+    ``x_next`` (the model dtype) receives ``rmsnorm(x) * w_next``, the next sublayer's input.
+    ``depth`` = (X, w, n) ends a layer of a depth-averaged model in the same launch: x is slot n - 1 of
+    the f32 stack X, slot n receives ``sum_{j<n} w[j] X[j]`` (as ``depth_mix``) and ``x_next`` is
+    normed from that; returns the slot handed on."""
     ext = _native(a)
     if ext is None:
-        return ref.resadd_norm(a, w_post, eps, x, w_next, x_next, b, wa, wb)
-    ext.resadd_norm(a, b, wa, wb, w_post, float(eps), x, w_next, x_next)
-    return x
+        ref.resadd_norm(a, w_post, eps, x, None if depth else w_next, None if depth else x_next, b, wa, wb)
+        return ref.depth_mix(depth[0], depth[1], depth[2], w_next, eps, x_next) if depth else x
+    if depth is None:
+        ext.resadd_norm(a, b, wa, wb, w_post, float(eps), x, w_next, x_next)
+        return x
+    X, w, n = depth
+    ext.resadd_norm(a, b, wa, wb, w_post, float(eps), x, w_next, x_next, X, w, int(n))
+    return X[n]
 
 
 def depth_mix(X: torch.Tensor, w: torch.Tensor, n: int, w_next: Optional[torch.Tensor] = None, eps: float = 0.0,

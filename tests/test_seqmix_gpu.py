@@ -202,6 +202,27 @@ def test_resadd_norm(dt, n, pair):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("pair", [False, True])
+def test_resadd_norm_with_depth_average(dt, pair):
+    """The layer-ending form: the residual update and the weighted sum over the stack in one launch."""
+    torch.manual_seed(8)
+    T, n = 7, 136
+    X1 = torch.randn(5, T, n, device=DEV)
+    X2 = X1.clone()
+    a, b = torch.randn(T, n, device=DEV).to(dt), torch.randn(T, n, device=DEV).to(dt)
+    wa, wb, wp, wn, dw = (torch.randn(k, device=DEV) for k in (n, n, n, n, 4))
+    kw = dict(b=b, wa=wa, wb=wb) if pair else {}
+    for slot in (1, 3):
+        h1, h2 = torch.empty(T, n, device=DEV, dtype=dt), torch.empty(T, n, device=DEV, dtype=dt)
+        o1 = seqmix.resadd_norm(a, wp, 1e-5, X1[slot], wn, h1, depth=(X1, dw, slot + 1), **kw)
+        o2 = ref.resadd_norm(a, wp, 1e-5, X2[slot], None, None, **kw)
+        o2 = ref.depth_mix(X2, dw, slot + 1, wn, 1e-5, h2)
+        torch.testing.assert_close(X1, X2, atol=2e-5, rtol=2e-5)
+        torch.testing.assert_close(o1, X1[slot + 1], atol=0, rtol=0)
+        torch.testing.assert_close(h1.float(), h2.float(), **tol(dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
 def test_depth_mix_and_gelu(dt):
     torch.manual_seed(3)
     X1 = torch.randn(6, 11, 72, device=DEV)
